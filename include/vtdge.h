@@ -1,0 +1,159 @@
+/*
+ * vtdge -- C ABI of the MI355X (gfx950) Dynamic Grained Encoder query path.
+ *
+ * One entry point per operator of the reference's native module `vtpack._C`
+ * (vtpack/layers/csrc/vision.cpp:9-29) that lies on the inference query path,
+ * plus the dense pieces of the transformer block that sit between them
+ * (LayerNorm, Linear) so a whole block runs without leaving the library.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in `_host`;
+ *   - the library never allocates, frees or synchronises: the caller owns all
+ *     buffers, every kernel is enqueued on `stream` (a hipStream_t, passed as
+ *     void* so the header needs no HIP include) and the call returns at once;
+ *   - tensors are dense row-major unless explicit element strides are given;
+ *   - `dtype` selects storage AND arithmetic flavour: VTDGE_F32 = fp32 storage,
+ *     fp32 arithmetic; VTDGE_BF16 = bf16 storage, fp32 accumulation, one
+ *     round-to-nearest-even on store;
+ *   - packed ("sparse") operands are [rows, C] matrices whose row count is only
+ *     known on the device after routing.  Such calls take `rows` (a host-side
+ *     upper bound: grid size, buffer capacity) and `rows_dev` (nullable device
+ *     pointer to the live int64 row count; when NULL, `rows` itself is live);
+ *   - return value: VTDGE_OK (0) or a negative VTDGE_ERR_*; vtdge_last_error()
+ *     gives a thread-local message.  No exceptions cross the ABI.
+ */
+#ifndef VTDGE_H
+#define VTDGE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VTDGE_OK 0
+#define VTDGE_ERR_ARG (-1)         /* NULL pointer, non-positive size, bad enum     */
+#define VTDGE_ERR_UNSUPPORTED (-2) /* valid request outside the built kernel family */
+#define VTDGE_ERR_LAUNCH (-3)      /* hipLaunchKernel / hipGetLastError failed      */
+
+#define VTDGE_F32 0
+#define VTDGE_BF16 1
+
+#define VTDGE_ACT_NONE 0
+#define VTDGE_ACT_GELU 1 /* exact erf GELU (torch.nn.GELU default) */
+
+#define VTDGE_MAX_SPLITS 8
+
+int vtdge_version(void);
+const char *vtdge_last_error(void);
+
+/* Router: region mean of the spatial tokens, Linear(C -> S), argmax.
+ * Replaces DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75).
+ *   x       [B, extra + H*W, C]      weight [S, C]      bias [S]
+ *   gate    [B, H/R, W/R, S] in `dtype` (nullable)      indices int64 [B, H/R, W/R]
+ * The mean is taken over the R x R window in dy-outer / dx-inner order in fp32;
+ * with VTDGE_BF16 the pooled value and the logits are rounded to bf16 as the
+ * reference's modules would, and the argmax (lowest index wins a tie) is taken
+ * on the rounded logits. */
+int vtdge_router(const void *x, const void *weight, const void *bias, void *gate, int64_t *indices,
+                 int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream);
+
+/* Gate indices -> packed query descriptors.
+ * Replaces grained_sample_index_to_patch
+ * (vtpack/layers/csrc/grained_sample/grained_sample.cu:302-345, kernel :146-196).
+ *   indices int64 [B, Hr, Wr]   splits int64 [S] (device, as in the reference)
+ *   patches int64 [capacity_rows, 4] rows = [sample, y0, x0, size]; extra-token
+ *           rows are [sample, -(e+1), 0, 1] (the reference leaves column 2 of
+ *           those rows unwritten; 0 is written here).  Nullable: lengths only.
+ *   offsets int64 [B+1] exclusive prefix of lengths (offsets[B] = total rows L)
+ *   lengths int64 [B]   (the reference returns these on the host; copying them
+ *           is the caller's business so that the fused path needs no sync)
+ * Rows past `capacity_rows` are never written.  Gate indices outside [0,S) are
+ * clamped (the reference reads out of bounds). */
+int vtdge_index_to_patch(const int64_t *indices, const int64_t *splits, int B, int Hr, int Wr, int S,
+                         int R, int extra, int64_t *patches, int64_t capacity_rows, int64_t *offsets,
+                         int64_t *lengths, void *stream);
+
+/* Every patch of every granularity (exported by the reference, unused by its
+ * models).  Replaces grained_sample_index_to_patch_dense (grained_sample.cu:347-433).
+ *   patches int64 [B * per_sample, 4], per_sample = extra + Hr*Wr*sum(splits^2)
+ *   splits_host: HOST pointer (the reference copies it to the host too, :401). */
+int vtdge_index_to_patch_dense(const int64_t *splits_host, int B, int Hr, int Wr, int S, int R, int extra,
+                               int64_t *patches, void *stream);
+
+/* Grained sampling ("compress"): one packed query row per patch = mean of its
+ * size x size token window (fp32 accumulation, dy outer / dx inner, one divide),
+ * or a copy of the extra token.
+ * Replaces grained_sample_compress (grained_sample.cu:198-239, kernel :31-69).
+ *   x [B, N, C]   patches [rows, 4]   out [rows, C]
+ * Optional fused LayerNorm of the (rounded) output row, as the block applies
+ * norm1 to the compressed queries (vtpack/models/dge/deit_dge.py:127):
+ *   ln_out [rows, C] nullable; ln_weight, ln_bias [C]. */
+int vtdge_compress(const void *x, const int64_t *patches, const int64_t *rows_dev, int64_t rows,
+                   void *out, void *ln_out, const void *ln_weight, const void *ln_bias, float ln_eps,
+                   int B, int N, int C, int W, int extra, int dtype, void *stream);
+
+/* Scatter back ("decompress"): every token covered by a patch receives
+ *   out[b,t,:] = (in[row,:] - sub[row,:]) + ref[b,t,:]
+ * with `sub` and `ref` each optional (NULL = term absent).
+ * Replaces grained_sample_decompress, both overloads (grained_sample.cu:241-300,
+ * kernels :71-144; ref == NULL is is_add_ref = false) and, with `sub`, the
+ * subtraction in DynamicGrainedEncoder.decompress (vtpack/layers/dge.py:88).
+ * In bf16 the difference is rounded to bf16 before the add, as the reference's
+ * separate elementwise op would.  Tokens no patch covers are left untouched. */
+int vtdge_decompress(const void *in, const void *sub, const int64_t *patches, const int64_t *rows_dev,
+                     int64_t rows, const void *ref, void *out, int B, int N, int C, int W, int extra,
+                     int dtype, void *stream);
+
+/* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
+ * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */
+int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out, const int64_t *rows_dev,
+                    int64_t rows, int C, float eps, int dtype, void *stream);
+
+/* Packed-M Linear: out[m, n] = act(sum_k A[m,k] * W[n,k] + bias[n]) + residual[m,n].
+ * The M dimension is the packed query set of all samples (weights are shared),
+ * which is what the reference's q / proj / fc1 / fc2 nn.Linear calls compute on
+ * [L, C] (vtpack/models/dge/deit_dge.py:72,96,38-44) and kv on [B*N, C] (:73).
+ *   A [rows, K] leading dim lda      W [N, K] dense      bias [N] nullable
+ *   residual [rows, N] leading dim ldr, nullable         out [rows, N] leading dim ldo
+ * MFMA kernel; K must be a multiple of 32 bytes worth of elements (8 fp32 / 16 bf16). */
+int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,
+                 int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K,
+                 int act, int dtype, void *stream);
+
+/* Sparse attention of packed queries against each sample's full K/V:
+ *   out[rows of sample i, head a] = softmax(scale * Q_i,a K_i,a^T) V_i,a
+ * Replaces batched_sparse_attention_forward
+ * (vtpack/layers/csrc/batched_sparse_gemm/batched_sparse_gemm.cu:219-305).
+ * All operands are addressed through element strides so that both the
+ * reference's contiguous [h, L, d] / [h, B, n, d] tensors and the un-permuted
+ * outputs of the q / kv Linears ([L, h*d] and [B, n, 2, h, d]) can be passed:
+ *   q(row, a, c)   = q[row*q_row_stride + a*q_head_stride + c]
+ *   k(i, t, a, c)  = k[i*kv_batch_stride + t*kv_tok_stride + a*kv_head_stride + c]  (same for v)
+ *   out(row, a, c) = out[row*o_row_stride + a*o_head_stride + c]
+ *   offsets int64 [B+1] (device) exclusive prefix of the per-sample query counts
+ *   max_rows_per_sample: host upper bound of any sample's query count (grid size)
+ * head_dim d must be 64 or 32. */
+int vtdge_sparse_attention(const void *q, int64_t q_row_stride, int64_t q_head_stride, const void *k,
+                           const void *v, int64_t kv_batch_stride, int64_t kv_tok_stride,
+                           int64_t kv_head_stride, const int64_t *offsets, void *out, int64_t o_row_stride,
+                           int64_t o_head_stride, int B, int h, int d, int n, int max_rows_per_sample,
+                           float scale, int dtype, void *stream);
+
+/* Per-sample variable-length batched matmul over heads.
+ * Replaces batched_sparse_gemm_forward and batched_sparse_gemm_v2_forward
+ * (batched_sparse_gemm.cu:150-195, :83-148):
+ *   a [h, La, ka], b [h, Lb, kb]; sample i uses rows a_offsets[i]..a_offsets[i+1]
+ *   of a and b_offsets[i]..b_offsets[i+1] of b, each optionally transposed in its
+ *   last two dims; out [h, out_rows, out_cols] is the concatenation along dim 1.
+ *   a_offsets, b_offsets int64 [B+1] on the device.
+ *   max_m: host upper bound of any sample's output row count (grid size). */
+int vtdge_batched_sparse_gemm(const void *a, const void *b, const int64_t *a_offsets, const int64_t *b_offsets,
+                              void *out, int B, int h, int64_t La, int ka, int64_t Lb, int kb, int trans_a,
+                              int trans_b, int64_t out_rows, int64_t out_cols, int64_t max_m, int dtype,
+                              void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VTDGE_H */

@@ -1,0 +1,284 @@
+"""GPU parity of every libvtdge operator against the CPU oracle, through the C ABI.
+
+Integer outputs (gate indices, query counts, patch descriptors) are compared bit-exactly;
+floating point within the tolerances stated in tests/util.py.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dge_oracle as orc
+from oracle import torch_ref
+from util import SPLITS, assert_close, bf16_round, randn, random_indices, rel_err, rng
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _t(a, dev, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    return t if dtype is None else t.to(dtype)
+
+
+# ------------------------------------------------------------------ index -> patch
+@pytest.mark.parametrize("B,Hr,Wr,extra,splits", [
+    (8, 4, 4, 1, [4, 2, 1]),      # config 1 geometry
+    (1, 1, 1, 1, [4, 2, 1]),
+    (3, 2, 3, 0, [4, 2, 1]),      # non-square, no extra token (PVT-like)
+    (5, 8, 8, 2, [4, 2, 1]),      # 512 px geometry, distilled-style 2 extra tokens
+    (33, 4, 4, 1, [2, 1]),
+    (7, 4, 4, 1, [1]),
+    (2, 20, 20, 1, [4, 2, 1]),    # > 256 regions per sample: several passes of the LDS scan
+    (1500, 4, 4, 1, [4, 2, 1]),   # > 1024 samples: several passes of the sample scan
+])
+def test_index_to_patch_bit_exact(dev, B, Hr, Wr, extra, splits):
+    from vtpack_amd import _C
+    R = max(splits)
+    idx = random_indices(B * 7 + Hr, B, Hr, Wr, S=len(splits))
+    want_p, want_l = orc.index_to_patch(idx, splits, R, extra)
+    got_p, got_l = _C.grained_sample_index_to_patch(_t(idx, dev), _t(np.array(splits, dtype=np.int64), dev), R, extra)
+    assert got_l.device.type == "cpu" and got_l.dtype == torch.int64
+    assert np.array_equal(got_l.numpy(), want_l)
+    assert got_p.shape == want_p.shape
+    assert np.array_equal(got_p.cpu().numpy(), want_p)
+
+
+def test_index_to_patch_uniform_gates(dev):
+    from vtpack_amd import _C
+    sp = _t(np.array(SPLITS, dtype=np.int64), dev)
+    for g in range(3):
+        idx = np.full((4, 4, 4), g, dtype=np.int64)
+        want_p, want_l = orc.index_to_patch(idx, SPLITS, 4, 1)
+        got_p, got_l = _C.grained_sample_index_to_patch(_t(idx, dev), sp, 4, 1)
+        assert np.array_equal(got_p.cpu().numpy(), want_p) and np.array_equal(got_l.numpy(), want_l)
+
+
+def test_index_to_patch_dense(dev):
+    from vtpack_amd import _C
+    idx = random_indices(3, 3, 4, 4)
+    want_p, want_l = orc.index_to_patch_dense(idx, SPLITS, 4, 1)
+    got_p, got_l = _C.grained_sample_index_to_patch_dense(_t(idx, dev), _t(np.array(SPLITS, dtype=np.int64), dev), 4, 1)
+    assert np.array_equal(got_p.cpu().numpy(), want_p) and np.array_equal(got_l.numpy(), want_l)
+
+
+# ------------------------------------------------------------------ compress / decompress
+GEOMS = [(8, 16, 16, 1, 192), (2, 32, 32, 1, 384), (3, 8, 12, 0, 64), (2, 16, 16, 2, 768)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,W,extra,C", GEOMS)
+def test_compress_bit_exact(dev, dtype, B, H, W, extra, C):
+    from vtpack_amd import _C
+    idx = random_indices(B + C, B, H // 4, W // 4)
+    patches, _ = orc.index_to_patch(idx, SPLITS, 4, extra)
+    x = randn(C + 1, B, extra + H * W, C)
+    if dtype == torch.bfloat16:
+        x = bf16_round(x)
+    want = orc.compress(x, patches, H, W, extra)
+    got = _C.grained_sample_compress(_t(x, dev, dtype), _t(patches, dev), H, W, extra)
+    assert got.dtype == dtype and tuple(got.shape) == want.shape
+    want_t = torch.from_numpy(want).to(dtype)       # one round-to-nearest-even on store
+    assert torch.equal(got.cpu(), want_t), f"max diff {rel_err(got.float(), want_t.float()):.3e}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("add_ref", [True, False])
+@pytest.mark.parametrize("B,H,W,extra,C", GEOMS)
+def test_decompress_bit_exact(dev, dtype, add_ref, B, H, W, extra, C):
+    from vtpack_amd import _C
+    idx = random_indices(B + C + 5, B, H // 4, W // 4)
+    patches, _ = orc.index_to_patch(idx, SPLITS, 4, extra)
+    d = randn(C + 2, patches.shape[0], C)
+    ref = randn(C + 3, B, extra + H * W, C)
+    if dtype == torch.bfloat16:
+        d, ref = bf16_round(d), bf16_round(ref)
+    want = torch.from_numpy(orc.decompress(d, patches, ref, H, W, extra, add_ref)).to(dtype)
+    got = _C.grained_sample_decompress(_t(d, dev, dtype), _t(patches, dev), _t(ref, dev, dtype), H, W, extra, add_ref)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decompress_fused_subtract(dev, dtype):
+    """out = (q - comp) + ref in one kernel == DynamicGrainedEncoder.decompress (dge.py:88 + scatter)."""
+    from vtpack_amd import ops
+    B, H, W, extra, C = 4, 16, 16, 1, 192
+    idx = random_indices(11, B, 4, 4)
+    patches, _ = orc.index_to_patch(idx, SPLITS, 4, extra)
+    q, comp = randn(1, patches.shape[0], C), randn(2, patches.shape[0], C)
+    ref = randn(3, B, extra + H * W, C)
+    if dtype == torch.bfloat16:
+        q, comp, ref = bf16_round(q), bf16_round(comp), bf16_round(ref)
+    delta = torch.from_numpy(q - comp).to(dtype).float().numpy()      # the reference rounds the difference
+    want = torch.from_numpy(orc.decompress(delta, patches, ref, H, W, extra, True)).to(dtype)
+    got = ops.decompress(_t(q, dev, dtype), _t(patches, dev), _t(ref, dev, dtype), W, extra, add_ref=True,
+                         sub=_t(comp, dev, dtype))
+    assert torch.equal(got.cpu(), want)
+
+
+def test_device_side_row_count(dev):
+    """Packed kernels stop at the row count held in device memory, not at the buffer capacity."""
+    from vtpack_amd import ops
+    B, H, W, extra, C = 4, 16, 16, 1, 192
+    idx = random_indices(5, B, 4, 4)
+    want_p, want_l = orc.index_to_patch(idx, SPLITS, 4, extra)
+    cap = B * (extra + H * W)
+    patches, offsets, lengths = ops.index_to_patch(_t(idx, dev), _t(np.array(SPLITS, dtype=np.int64), dev), 4, extra,
+                                                   capacity=cap)
+    L = int(want_l.sum())
+    assert np.array_equal(offsets.cpu().numpy(), np.concatenate([[0], np.cumsum(want_l)]))
+    assert np.array_equal(patches[:L].cpu().numpy(), want_p)
+    x = randn(9, B, extra + H * W, C)
+    sentinel = 12345.0
+    out = torch.full((cap, C), sentinel, device=dev)
+    from vtpack_amd._lib import call, ptr, stream_ptr, F32
+    call("vtdge_compress", ptr(_t(x, dev)), ptr(patches), ptr(offsets[B:]), cap, ptr(out), 0, 0, 0, 0.0, B,
+         extra + H * W, C, W, extra, F32, stream_ptr())
+    assert torch.equal(out[:L].cpu(), torch.from_numpy(orc.compress(x, want_p, H, W, extra)))
+    assert bool((out[L:] == sentinel).all())
+
+
+# ------------------------------------------------------------------ router
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,W,extra,C", [(8, 16, 16, 1, 192), (4, 32, 32, 1, 384), (3, 8, 12, 0, 64)])
+def test_router_gate_and_indices(dev, dtype, B, H, W, extra, C):
+    from vtpack_amd import ops
+    x = randn(21, B, extra + H * W, C)
+    w = randn(22, 3, C) * 0.3
+    b = randn(23, 3) * 0.1
+    if dtype == torch.bfloat16:
+        x, w, b = bf16_round(x), bf16_round(w), bf16_round(b)
+    want = torch_ref.router_gate(torch.from_numpy(x), H, W, torch.from_numpy(w), torch.from_numpy(b), 4)
+    gate, indices = ops.router(_t(x, dev, dtype), _t(w, dev, dtype), _t(b, dev, dtype), H, W, 4)
+    assert_close(gate.float(), want, dtype, "gate logits")
+    # gate choices must be identical wherever the decision is not a numerical tie of the oracle's own logits
+    top2 = want.topk(2, dim=-1).values
+    margin = (top2[..., 0] - top2[..., 1])
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    decided = margin > tol
+    assert decided.float().mean() > 0.9
+    assert torch.equal(indices.cpu()[decided], want.argmax(-1)[decided])
+    # and the kernel's indices are exactly the argmax of the kernel's own (rounded) logits, lowest index on ties
+    assert torch.equal(indices.cpu(), gate.float().cpu().argmax(-1))
+
+
+# ------------------------------------------------------------------ layernorm / linear
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,C", [(1, 192), (257, 384), (1000, 768), (33, 64)])
+def test_layernorm(dev, dtype, rows, C):
+    from vtpack_amd import ops
+    x, w, b = randn(31, rows, C) * 2 + 0.5, randn(32, C) * 0.2 + 1, randn(33, C) * 0.1
+    if dtype == torch.bfloat16:
+        x, w, b = bf16_round(x), bf16_round(w), bf16_round(b)
+    want = torch.nn.functional.layer_norm(torch.from_numpy(x), (C,), torch.from_numpy(w), torch.from_numpy(b), 1e-6)
+    got = ops.layernorm(_t(x, dev, dtype), _t(w, dev, dtype), _t(b, dev, dtype), 1e-6)
+    assert_close(got.float(), want, dtype, "layernorm")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 192, 192), (904, 576, 192), (257, 384, 384), (1000, 1536, 384),
+                                     (300, 384, 1536), (129, 1000, 192), (64, 72, 40)])
+@pytest.mark.parametrize("epi", ["plain", "bias", "bias_gelu", "bias_res"])
+def test_linear(dev, dtype, M, N, K, epi):
+    from vtpack_amd import ops
+    a, w = randn(41, M, K), randn(42, N, K) * 0.02   # the isolated-GEMM config: A ~ N(0,1), W ~ N(0,0.02)
+    bias, res = randn(43, N) * 0.1, randn(44, M, N)
+    if dtype == torch.bfloat16:
+        a, w, bias, res = bf16_round(a), bf16_round(w), bf16_round(bias), bf16_round(res)
+    want = torch.from_numpy(a).double() @ torch.from_numpy(w).double().T
+    if epi != "plain":
+        want = want + torch.from_numpy(bias).double()
+    if epi == "bias_gelu":
+        want = torch.nn.functional.gelu(want)
+    if epi == "bias_res":
+        want = want + torch.from_numpy(res).double()
+    got = ops.linear(_t(a, dev, dtype), _t(w, dev, dtype), None if epi == "plain" else _t(bias, dev, dtype),
+                     _t(res, dev, dtype) if epi == "bias_res" else None, act="gelu" if epi == "bias_gelu" else "none")
+    assert_close(got.float(), want, dtype, f"linear {epi}")
+
+
+def test_linear_device_rows(dev):
+    from vtpack_amd import ops
+    M, N, K, live = 700, 384, 192, 333
+    a, w = randn(51, M, K), randn(52, N, K) * 0.05
+    rows_dev = torch.tensor([live], dtype=torch.int64, device=dev)
+    out = torch.full((M, N), 7.0, device=dev)
+    ops.linear(_t(a, dev), _t(w, dev), rows_dev=rows_dev, out=out)
+    want = torch.from_numpy(a[:live]).double() @ torch.from_numpy(w).double().T
+    assert rel_err(out[:live], want) <= 1e-5
+    assert bool((out[live:] == 7.0).all())
+
+
+# ------------------------------------------------------------------ attention / sparse gemm
+def _lengths(seed, B, lo, hi):
+    return rng(seed).randint(lo, hi + 1, size=B).astype(np.int64)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,h,d,n,lo,hi", [(8, 3, 64, 257, 17, 257), (2, 6, 64, 1025, 65, 400), (3, 2, 32, 50, 1, 70),
+                                             (4, 1, 64, 128, 128, 128), (2, 2, 64, 129, 1, 3)])
+def test_sparse_attention(dev, dtype, B, h, d, n, lo, hi):
+    from vtpack_amd import _C
+    lengths = _lengths(61 + n, B, lo, hi)
+    L = int(lengths.sum())
+    q, k, v = randn(62, h, L, d), randn(63, h, B, n, d), randn(64, h, B, n, d)
+    if dtype == torch.bfloat16:
+        q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+    scale = d ** -0.5
+    want = orc.attention(q, k, v, lengths, scale)
+    got = _C.batched_sparse_attention_forward(_t(q, dev, dtype), _t(k, dev, dtype), _t(v, dev, dtype),
+                                              torch.from_numpy(lengths), scale)
+    assert got.shape == (h, L, d)
+    assert_close(got.float(), want, dtype, "sparse attention")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sparse_attention_strided_kv(dev, dtype):
+    """q straight from the q Linear ([L, h*d]) and k, v as views of the kv Linear output ([B, n, 2, h, d])."""
+    from vtpack_amd import ops
+    B, h, d, n = 4, 3, 64, 257
+    C = h * d
+    lengths = _lengths(71, B, 17, 257)
+    L = int(lengths.sum())
+    q, kv = randn(72, L, C), randn(73, B, n, 2 * C)
+    if dtype == torch.bfloat16:
+        q, kv = bf16_round(q), bf16_round(kv)
+    qh = q.reshape(L, h, d).transpose(1, 0, 2)
+    kvh = kv.reshape(B, n, 2, h, d).transpose(2, 3, 0, 1, 4)
+    want = orc.attention(qh, kvh[0], kvh[1], lengths, d ** -0.5).transpose(1, 0, 2).reshape(L, C)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(lengths)])).to(dev)
+    kvt = _t(kv, dev, dtype)
+    got = ops.sparse_attention(_t(q, dev, dtype), kvt[:, :, :C], kvt[:, :, C:], off, d ** -0.5, h, int(lengths.max()))
+    assert_close(got.float(), want, dtype, "strided sparse attention")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+def test_batched_sparse_gemm(dev, dtype, ta, tb):
+    from vtpack_amd import _C
+    B, h, d, n = 5, 3, 64, 70
+    la = _lengths(81, B, 3, 90)
+    if not ta and tb:        # Q K^T: a [h,La,d], b [h,B*n,d]
+        lb = np.full(B, n, dtype=np.int64)
+        a, b = randn(82, h, int(la.sum()), d), randn(83, h, int(lb.sum()), d)
+    elif not ta and not tb:  # P V: a [h,La,n], b [h,B*n,d]
+        lb = np.full(B, n, dtype=np.int64)
+        a, b = randn(82, h, int(la.sum()), n), randn(83, h, int(lb.sum()), d)
+    elif ta and not tb:      # A^T B: a [h,La,ka], b [h,La,kb]
+        lb = la.copy()
+        a, b = randn(82, h, int(la.sum()), 48), randn(83, h, int(lb.sum()), d)
+    else:                    # A^T B^T: a [h,La,ka] -> [ka,la]; b [h,Lb,kb] with kb == la, so equal lengths
+        la = np.full(B, 40, dtype=np.int64)
+        lb = np.full(B, 24, dtype=np.int64)
+        a, b = randn(82, h, int(la.sum()), 48), randn(83, h, int(lb.sum()), 40)
+    if dtype == torch.bfloat16:
+        a, b = bf16_round(a), bf16_round(b)
+    want = orc.sparse_gemm(a, b, la, lb, ta, tb)
+    for fn in (_C.batched_sparse_gemm_forward, _C.batched_sparse_gemm_v2_forward):
+        got = fn(_t(a, dev, dtype), _t(b, dev, dtype), torch.from_numpy(la), torch.from_numpy(lb), ta, tb)
+        assert tuple(got.shape) == want.shape
+        if dtype == torch.float32:
+            assert rel_err(got, want) <= 1e-5
+        else:
+            # bf16 output of sums of ~64 products of N(0,1) values: one bf16 rounding of |x| <~ 40
+            assert rel_err(got.float(), want) <= 2 ** -8

@@ -1,0 +1,136 @@
+// Shared device/host helpers of the vtdge kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/vtdge.h"
+
+namespace vtdge {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+#define VT_REQUIRE(cond, code, ...)  \
+    do {                             \
+        if (!(cond)) {               \
+            set_error(__VA_ARGS__);  \
+            return (code);           \
+        }                            \
+    } while (0)
+
+// ---------------------------------------------------------------- types
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round-to-nearest-even, NaN stays NaN (quiet)
+__device__ __forceinline__ bf16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Storage-type traits: a 16-byte vector of T holds VEC elements.
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ float load(const float *p) { return *p; }
+    static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+    static __device__ __forceinline__ float round(float v) { return v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float *f)
+    {
+        f[0] = __uint_as_float(r.x); f[1] = __uint_as_float(r.y);
+        f[2] = __uint_as_float(r.z); f[3] = __uint_as_float(r.w);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f)
+    {
+        u32x4 r;
+        r.x = __float_as_uint(f[0]); r.y = __float_as_uint(f[1]);
+        r.z = __float_as_uint(f[2]); r.w = __float_as_uint(f[3]);
+        return r;
+    }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ float load(const bf16_t *p) { return bf16_to_f32(*p); }
+    static __device__ __forceinline__ void store(bf16_t *p, float v) { *p = f32_to_bf16(v); }
+    static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float *f)
+    {
+        f[0] = bf16lo(r.x); f[1] = bf16hi(r.x); f[2] = bf16lo(r.y); f[3] = bf16hi(r.y);
+        f[4] = bf16lo(r.z); f[5] = bf16hi(r.z); f[6] = bf16lo(r.w); f[7] = bf16hi(r.w);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f)
+    {
+        u32x4 r;
+        r.x = pack_bf16x2(f[0], f[1]); r.y = pack_bf16x2(f[2], f[3]);
+        r.z = pack_bf16x2(f[4], f[5]); r.w = pack_bf16x2(f[6], f[7]);
+        return r;
+    }
+};
+
+// ---------------------------------------------------------------- MFMA
+// One 32-byte K-slab of a 32x32 output block: lane (r = lane%32, g = lane/32)
+// supplies bytes [16g, 16g+16) of row r of each operand.
+template <typename T> struct Slab;
+template <> struct Slab<bf16_t> {
+    static __device__ __forceinline__ void mma(const u32x4 &a, const u32x4 &b, f32x16 &c)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                    0, 0, 0);
+    }
+};
+template <> struct Slab<float> {
+    static __device__ __forceinline__ void mma(const u32x4 &a, const u32x4 &b, f32x16 &c)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+    }
+};
+
+// ---------------------------------------------------------------- wave ops
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ int64_t live_rows(const int64_t *rows_dev, int64_t rows)
+{
+    if (rows_dev == nullptr) return rows;
+    int64_t r = *rows_dev;
+    return r < rows ? r : rows;
+}
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace vtdge

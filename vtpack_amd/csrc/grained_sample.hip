@@ -1,0 +1,648 @@
+// Grained sampling kernels for gfx950: router, index->patch compaction,
+// compress (gather + window mean) and decompress (scatter back).
+//
+// All four are HBM-bandwidth or latency bound.  The element kernels give one
+// 64-lane wavefront to one packed query row and move 16 bytes per lane, so a
+// row of C channels is read/written with fully coalesced 16-byte accesses.
+#include "common.h"
+
+namespace vtdge {
+
+constexpr int ROWS_PER_BLOCK = 4;  // one wave per row, 256 threads
+constexpr int MAX_IT = 3;          // 16-byte vectors per lane: C <= 64*3*VEC
+
+// ------------------------------------------------------------------ router
+// One wave per region.  Replaces AvgPool2d(R,R) -> Linear(C,S) -> argmax
+// (vtpack/layers/dge.py:145-150, :75).
+template <typename T>
+__global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, const T *__restrict__ weight,
+                                                      const T *__restrict__ bias, T *__restrict__ gate,
+                                                      int64_t *__restrict__ indices, int B, int H, int W,
+                                                      int C, int extra, int R, int S)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int Hr = H / R, Wr = W / R;
+    const int64_t region = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    if (region >= (int64_t)B * Hr * Wr) return;
+    const int b = (int)(region / (Hr * Wr));
+    const int rr = (int)(region % (Hr * Wr));
+    const int ry = rr / Wr, rx = rr % Wr;
+    const int N = extra + H * W;
+    const int nvec = C / VEC;
+    const T *xb = x + (int64_t)b * N * C;
+    const float area = (float)(R * R);
+
+    float part[VTDGE_MAX_SPLITS];
+#pragma unroll
+    for (int s = 0; s < VTDGE_MAX_SPLITS; s++) part[s] = 0.f;
+
+    for (int v = lane; v < nvec; v += WAVE) {
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+        for (int dy = 0; dy < R; dy++) {
+            for (int dx = 0; dx < R; dx++) {
+                const int tok = (ry * R + dy) * W + rx * R + dx + extra;
+                u32x4 raw = *reinterpret_cast<const u32x4 *>(xb + (int64_t)tok * C + v * VEC);
+                float f[VEC];
+                Elem<T>::unpack(raw, f);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) acc[i] += f[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = Elem<T>::round(acc[i] / area);
+#pragma unroll
+        for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
+            if (s < S) {
+                u32x4 raw = *reinterpret_cast<const u32x4 *>(weight + (int64_t)s * C + v * VEC);
+                float w[VEC];
+                Elem<T>::unpack(raw, w);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) part[s] += acc[i] * w[i];
+            }
+        }
+    }
+    float best = 0.f;
+    int best_s = 0;
+#pragma unroll
+    for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
+        if (s < S) {
+            float logit = wave_sum(part[s]) + Elem<T>::load(bias + s);
+            logit = Elem<T>::round(logit);
+            if (gate != nullptr && lane == 0) Elem<T>::store(gate + region * S + s, logit);
+            if (s == 0 || logit > best) {  // strict >: lowest index wins a tie
+                best = logit;
+                best_s = s;
+            }
+        }
+    }
+    if (lane == 0) indices[region] = best_s;
+}
+
+// ------------------------------------------------------------ index->patch
+// Step 1 (single workgroup): per-sample query counts and their exclusive scan.
+// Counts: one wave per sample, lanes over regions, wave reduction.
+// Scan: 1024 samples per pass, wave-level shuffles + LDS for the wave totals.
+__global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *__restrict__ indices,
+                                                                 const int64_t *__restrict__ splits, int B,
+                                                                 int nreg, int S, int extra,
+                                                                 int64_t *__restrict__ offsets,
+                                                                 int64_t *__restrict__ lengths)
+{
+    __shared__ int64_t wave_tot[16];
+    __shared__ int64_t carry_s;
+    __shared__ int sq[VTDGE_MAX_SPLITS];
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    if (threadIdx.x < VTDGE_MAX_SPLITS) {
+        int ps = threadIdx.x < S ? (int)splits[threadIdx.x] : 0;
+        sq[threadIdx.x] = ps * ps;
+    }
+    if (threadIdx.x == 0) carry_s = 0;
+    __syncthreads();
+    for (int b = wid; b < B; b += 16) {
+        int cnt = 0;
+        for (int r = lane; r < nreg; r += WAVE) {
+            int64_t g = indices[(int64_t)b * nreg + r];
+            g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+            cnt += sq[g];
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, WAVE);
+        if (lane == 0) lengths[b] = (int64_t)cnt + extra;
+    }
+    __syncthreads();  // lengths[] written by this block are visible to it
+    for (int base = 0; base < B; base += 1024) {
+        const int b = base + threadIdx.x;
+        int64_t v = b < B ? lengths[b] : 0;
+        int64_t inc = v;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            int64_t up = __shfl_up(inc, o, WAVE);
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) wave_tot[wid] = inc;
+        __syncthreads();
+        int64_t before = carry_s;
+        for (int w = 0; w < wid; w++) before += wave_tot[w];
+        if (b < B) offsets[b] = before + inc - v;
+        __syncthreads();
+        if (threadIdx.x == 1023) carry_s = before + inc;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) offsets[B] = carry_s;
+}
+
+// Step 2: one workgroup per sample.  The per-region query counts go through an
+// LDS-staged wavefront prefix sum (256 regions per pass); each thread then
+// emits the descriptors of its own region at offsets[b] + extra + prefix.
+__global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restrict__ indices,
+                                                           const int64_t *__restrict__ splits,
+                                                           const int64_t *__restrict__ offsets, int Hr, int Wr,
+                                                           int S, int R, int extra, int64_t *__restrict__ patches,
+                                                           int64_t capacity)
+{
+    __shared__ int wave_tot[4];
+    __shared__ int carry_s;
+    __shared__ int split_s[VTDGE_MAX_SPLITS];
+    const int b = blockIdx.x;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int nreg = Hr * Wr;
+    if (threadIdx.x < VTDGE_MAX_SPLITS) split_s[threadIdx.x] = threadIdx.x < S ? (int)splits[threadIdx.x] : 1;
+    if (threadIdx.x == 0) carry_s = 0;
+    __syncthreads();
+    const int64_t row0 = offsets[b];
+    for (int e = threadIdx.x; e < extra; e += 256) {
+        const int64_t row = row0 + e;
+        if (row < capacity) {
+            int64_t *p = patches + 4 * row;
+            p[0] = b; p[1] = -(int64_t)e - 1; p[2] = 0; p[3] = 1;
+        }
+    }
+    for (int base = 0; base < nreg; base += 256) {
+        const int r = base + threadIdx.x;
+        int ps = 0;
+        if (r < nreg) {
+            int64_t g = indices[(int64_t)b * nreg + r];
+            g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+            ps = split_s[g];
+        }
+        const int cnt = ps * ps;
+        int inc = cnt;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            int up = __shfl_up(inc, o, WAVE);
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) wave_tot[wid] = inc;
+        __syncthreads();
+        int before = carry_s;
+        for (int w = 0; w < wid; w++) before += wave_tot[w];
+        if (r < nreg) {
+            const int ry = r / Wr, rx = r % Wr;
+            const int step = R / ps;
+            int64_t row = row0 + extra + before + inc - cnt;
+            for (int dy = 0; dy < ps; dy++) {
+                for (int dx = 0; dx < ps; dx++, row++) {
+                    if (row < capacity) {
+                        int64_t *p = patches + 4 * row;
+                        p[0] = b;
+                        p[1] = (int64_t)ry * R + dy * step;
+                        p[2] = (int64_t)rx * R + dx * step;
+                        p[3] = step;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 255) carry_s = before + inc;
+        __syncthreads();
+    }
+}
+
+struct DenseSplits {
+    int n;
+    int ps[VTDGE_MAX_SPLITS];
+};
+
+// One thread per descriptor; closed-form enumeration (grained_sample.cu:347-391).
+__global__ __launch_bounds__(256) void patch_dense_kernel(DenseSplits sp, int B, int Hr, int Wr, int R, int extra,
+                                                           int per_sample, int64_t *__restrict__ patches)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)B * per_sample) return;
+    const int b = (int)(idx / per_sample);
+    int j = (int)(idx % per_sample);
+    int64_t *p = patches + 4 * idx;
+    if (j < extra) {
+        p[0] = b; p[1] = -(int64_t)j - 1; p[2] = 0; p[3] = 1;
+        return;
+    }
+    j -= extra;
+    for (int s = 0; s < sp.n; s++) {
+        const int ps = sp.ps[s];
+        const int len = Hr * Wr * ps * ps;
+        if (j < len) {
+            const int step = R / ps;
+            p[0] = b;
+            p[1] = (int64_t)(j / (Wr * ps)) * step;
+            p[2] = (int64_t)(j % (Wr * ps)) * step;
+            p[3] = step;
+            return;
+        }
+        j -= len;
+    }
+}
+
+// ---------------------------------------------------------------- compress
+template <typename T, int SZ>
+__device__ __forceinline__ void window_sum(const T *__restrict__ base, int W, int C, int sz,
+                                           float (&acc)[Elem<T>::VEC])
+{
+    constexpr int VEC = Elem<T>::VEC;
+    if constexpr (SZ > 0) {
+        u32x4 raw[SZ * SZ];
+#pragma unroll
+        for (int dy = 0; dy < SZ; dy++)
+#pragma unroll
+            for (int dx = 0; dx < SZ; dx++)
+                raw[dy * SZ + dx] = *reinterpret_cast<const u32x4 *>(base + ((int64_t)dy * W + dx) * C);
+#pragma unroll
+        for (int i = 0; i < SZ * SZ; i++) {
+            float f[VEC];
+            Elem<T>::unpack(raw[i], f);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) acc[c] += f[c];
+        }
+    } else {
+        for (int dy = 0; dy < sz; dy++)
+            for (int dx = 0; dx < sz; dx++) {
+                u32x4 raw = *reinterpret_cast<const u32x4 *>(base + ((int64_t)dy * W + dx) * C);
+                float f[VEC];
+                Elem<T>::unpack(raw, f);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc[c] += f[c];
+            }
+    }
+}
+
+template <typename T, bool LN>
+__global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, const int64_t *__restrict__ patches,
+                                                        const int64_t *__restrict__ rows_dev, int64_t rows,
+                                                        T *__restrict__ out, T *__restrict__ ln_out,
+                                                        const T *__restrict__ ln_w, const T *__restrict__ ln_b,
+                                                        float eps, int N, int C, int W, int extra)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    if (row >= live_rows(rows_dev, rows)) return;
+    const int64_t *p = patches + 4 * row;
+    const int64_t b = p[0], y0 = p[1], x0 = p[2];
+    const int sz = (int)p[3];
+    const int nvec = C / VEC;
+    const T *xb = x + b * (int64_t)N * C;
+
+    float vals[MAX_IT][VEC];
+#pragma unroll
+    for (int it = 0; it < MAX_IT; it++) {
+        const int v = it * WAVE + lane;
+        if (v < nvec) {
+            float acc[VEC];
+            if (y0 < 0) {
+                u32x4 raw = *reinterpret_cast<const u32x4 *>(xb + (-y0 - 1) * (int64_t)C + v * VEC);
+                Elem<T>::unpack(raw, acc);
+            } else {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc[c] = 0.f;
+                const T *base = xb + ((y0 * W + x0 + extra) * (int64_t)C + v * VEC);
+                if (sz == 1) window_sum<T, 1>(base, W, C, sz, acc);
+                else if (sz == 2) window_sum<T, 2>(base, W, C, sz, acc);
+                else if (sz == 4) window_sum<T, 4>(base, W, C, sz, acc);
+                else window_sum<T, 0>(base, W, C, sz, acc);
+                const float area = (float)(sz * sz);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc[c] = acc[c] / area;
+            }
+            *reinterpret_cast<u32x4 *>(out + row * (int64_t)C + v * VEC) = Elem<T>::pack(acc);
+            if constexpr (LN) {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) vals[it][c] = Elem<T>::round(acc[c]);
+            }
+        } else if constexpr (LN) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) vals[it][c] = 0.f;
+        }
+    }
+    if constexpr (LN) {
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < MAX_IT; it++)
+#pragma unroll
+            for (int c = 0; c < VEC; c++) s += vals[it][c];
+        const float mean = wave_sum(s) / (float)C;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < MAX_IT; it++) {
+            if (it * WAVE + lane < nvec) {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    const float dlt = vals[it][c] - mean;
+                    q += dlt * dlt;
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+#pragma unroll
+        for (int it = 0; it < MAX_IT; it++) {
+            const int v = it * WAVE + lane;
+            if (v < nvec) {
+                float w[VEC], bb[VEC], y[VEC];
+                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ln_w + v * VEC), w);
+                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ln_b + v * VEC), bb);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) y[c] = (vals[it][c] - mean) * rstd * w[c] + bb[c];
+                *reinterpret_cast<u32x4 *>(ln_out + row * (int64_t)C + v * VEC) = Elem<T>::pack(y);
+            }
+        }
+    }
+}
+
+// -------------------------------------------------------------- decompress
+template <typename T, int SZ, bool ADD>
+__device__ __forceinline__ void window_store(const T *__restrict__ ref, T *__restrict__ dst, int W, int C, int sz,
+                                             const float (&d)[Elem<T>::VEC])
+{
+    constexpr int VEC = Elem<T>::VEC;
+    if constexpr (SZ > 0) {
+        u32x4 raw[SZ * SZ];
+        if constexpr (ADD) {
+#pragma unroll
+            for (int dy = 0; dy < SZ; dy++)
+#pragma unroll
+                for (int dx = 0; dx < SZ; dx++)
+                    raw[dy * SZ + dx] = *reinterpret_cast<const u32x4 *>(ref + ((int64_t)dy * W + dx) * C);
+        }
+#pragma unroll
+        for (int dy = 0; dy < SZ; dy++)
+#pragma unroll
+            for (int dx = 0; dx < SZ; dx++) {
+                float o[VEC];
+                if constexpr (ADD) {
+                    float r[VEC];
+                    Elem<T>::unpack(raw[dy * SZ + dx], r);
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) o[c] = d[c] + r[c];
+                } else {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) o[c] = d[c];
+                }
+                *reinterpret_cast<u32x4 *>(dst + ((int64_t)dy * W + dx) * C) = Elem<T>::pack(o);
+            }
+    } else {
+        for (int dy = 0; dy < sz; dy++)
+            for (int dx = 0; dx < sz; dx++) {
+                float o[VEC];
+                if constexpr (ADD) {
+                    float r[VEC];
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + ((int64_t)dy * W + dx) * C), r);
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) o[c] = d[c] + r[c];
+                } else {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) o[c] = d[c];
+                }
+                *reinterpret_cast<u32x4 *>(dst + ((int64_t)dy * W + dx) * C) = Elem<T>::pack(o);
+            }
+    }
+}
+
+template <typename T, bool SUB, bool ADD>
+__global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ in, const T *__restrict__ sub,
+                                                          const int64_t *__restrict__ patches,
+                                                          const int64_t *__restrict__ rows_dev, int64_t rows,
+                                                          const T *__restrict__ ref, T *__restrict__ out, int N,
+                                                          int C, int W, int extra)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    if (row >= live_rows(rows_dev, rows)) return;
+    const int64_t *p = patches + 4 * row;
+    const int64_t b = p[0], y0 = p[1], x0 = p[2];
+    const int sz = (int)p[3];
+    const int nvec = C / VEC;
+    for (int v = lane; v < nvec; v += WAVE) {
+        float d[VEC];
+        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(in + row * (int64_t)C + v * VEC), d);
+        if constexpr (SUB) {
+            float s[VEC];
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(sub + row * (int64_t)C + v * VEC), s);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) d[c] = Elem<T>::round(d[c] - s[c]);
+        }
+        const int64_t tok = y0 < 0 ? (-y0 - 1) : (y0 * W + x0 + extra);
+        const int64_t off = (b * N + tok) * (int64_t)C + v * VEC;
+        const T *r = ADD ? ref + off : nullptr;
+        T *o = out + off;
+        if (y0 < 0 || sz == 1) window_store<T, 1, ADD>(r, o, W, C, 1, d);
+        else if (sz == 2) window_store<T, 2, ADD>(r, o, W, C, sz, d);
+        else if (sz == 4) window_store<T, 4, ADD>(r, o, W, C, sz, d);
+        else window_store<T, 0, ADD>(r, o, W, C, sz, d);
+    }
+}
+
+// --------------------------------------------------------------- layernorm
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                         const T *__restrict__ bsrc, T *__restrict__ out,
+                                                         const int64_t *__restrict__ rows_dev, int64_t rows, int C,
+                                                         float eps)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    if (row >= live_rows(rows_dev, rows)) return;
+    const int nvec = C / VEC;
+    float vals[MAX_IT][VEC];
+    float s = 0.f;
+#pragma unroll
+    for (int it = 0; it < MAX_IT; it++) {
+        const int v = it * WAVE + lane;
+        if (v < nvec) {
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(x + row * (int64_t)C + v * VEC), vals[it]);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) s += vals[it][c];
+        }
+    }
+    const float mean = wave_sum(s) / (float)C;
+    float q = 0.f;
+#pragma unroll
+    for (int it = 0; it < MAX_IT; it++) {
+        if (it * WAVE + lane < nvec) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float dlt = vals[it][c] - mean;
+                q += dlt * dlt;
+            }
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+#pragma unroll
+    for (int it = 0; it < MAX_IT; it++) {
+        const int v = it * WAVE + lane;
+        if (v < nvec) {
+            float ww[VEC], bb[VEC], y[VEC];
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(w + v * VEC), ww);
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(bsrc + v * VEC), bb);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) y[c] = (vals[it][c] - mean) * rstd * ww[c] + bb[c];
+            *reinterpret_cast<u32x4 *>(out + row * (int64_t)C + v * VEC) = Elem<T>::pack(y);
+        }
+    }
+}
+
+// ------------------------------------------------------------- host side
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename T> static int elem_vec() { return Elem<T>::VEC; }
+
+static int check_channels(int C, int dtype, const char *who)
+{
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(dtype == VTDGE_F32 || dtype == VTDGE_BF16, VTDGE_ERR_ARG, "%s: unknown dtype %d", who, dtype);
+    VT_REQUIRE(C > 0 && C % vec == 0, VTDGE_ERR_UNSUPPORTED, "%s: C=%d must be a positive multiple of %d", who, C,
+               vec);
+    return VTDGE_OK;
+}
+
+}  // namespace vtdge
+
+using namespace vtdge;
+
+extern "C" int vtdge_router(const void *x, const void *weight, const void *bias, void *gate, int64_t *indices,
+                            int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream)
+{
+    VT_REQUIRE(x && weight && bias && indices, VTDGE_ERR_ARG, "router: NULL operand");
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && R > 0 && extra >= 0, VTDGE_ERR_ARG, "router: bad sizes");
+    VT_REQUIRE(H % R == 0 && W % R == 0, VTDGE_ERR_ARG, "router: H=%d, W=%d not multiples of region %d", H, W, R);
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "router: S=%d outside [1,%d]", S,
+               VTDGE_MAX_SPLITS);
+    if (int rc = check_channels(C, dtype, "router")) return rc;
+    VT_REQUIRE(aligned16(x) && aligned16(weight), VTDGE_ERR_ARG, "router: operands must be 16-byte aligned");
+    const int64_t regions = (int64_t)B * (H / R) * (W / R);
+    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_F32)
+        router_kernel<float><<<grid, block, 0, st>>>((const float *)x, (const float *)weight, (const float *)bias,
+                                                     (float *)gate, indices, B, H, W, C, extra, R, S);
+    else
+        router_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t *)x, (const bf16_t *)weight,
+                                                      (const bf16_t *)bias, (bf16_t *)gate, indices, B, H, W, C,
+                                                      extra, R, S);
+    return check_launch("router");
+}
+
+extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *splits, int B, int Hr, int Wr, int S,
+                                    int R, int extra, int64_t *patches, int64_t capacity_rows, int64_t *offsets,
+                                    int64_t *lengths, void *stream)
+{
+    VT_REQUIRE(indices && splits && offsets && lengths, VTDGE_ERR_ARG, "index_to_patch: NULL operand");
+    VT_REQUIRE(B > 0 && Hr > 0 && Wr > 0 && R > 0 && extra >= 0, VTDGE_ERR_ARG, "index_to_patch: bad sizes");
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "index_to_patch: S=%d outside [1,%d]", S,
+               VTDGE_MAX_SPLITS);
+    VT_REQUIRE(patches == nullptr || capacity_rows >= 0, VTDGE_ERR_ARG, "index_to_patch: negative capacity");
+    hipStream_t st = (hipStream_t)stream;
+    patch_count_scan_kernel<<<1, 1024, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, offsets, lengths);
+    if (int rc = check_launch("index_to_patch(count+scan)")) return rc;
+    if (patches != nullptr) {
+        patch_write_kernel<<<B, 256, 0, st>>>(indices, splits, offsets, Hr, Wr, S, R, extra, patches,
+                                              capacity_rows);
+        return check_launch("index_to_patch(write)");
+    }
+    return VTDGE_OK;
+}
+
+extern "C" int vtdge_index_to_patch_dense(const int64_t *splits_host, int B, int Hr, int Wr, int S, int R,
+                                          int extra, int64_t *patches, void *stream)
+{
+    VT_REQUIRE(splits_host && patches, VTDGE_ERR_ARG, "index_to_patch_dense: NULL operand");
+    VT_REQUIRE(B > 0 && Hr > 0 && Wr > 0 && R > 0 && extra >= 0, VTDGE_ERR_ARG, "index_to_patch_dense: bad sizes");
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "index_to_patch_dense: S=%d", S);
+    DenseSplits sp;
+    sp.n = S;
+    int per = extra;
+    for (int s = 0; s < S; s++) {
+        VT_REQUIRE(splits_host[s] > 0 && R % splits_host[s] == 0, VTDGE_ERR_ARG,
+                   "index_to_patch_dense: split %lld does not divide region %d", (long long)splits_host[s], R);
+        sp.ps[s] = (int)splits_host[s];
+        per += sp.ps[s] * sp.ps[s] * Hr * Wr;
+    }
+    const int64_t total = (int64_t)B * per;
+    patch_dense_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(sp, B, Hr, Wr, R, extra,
+                                                                                        per, patches);
+    return check_launch("index_to_patch_dense");
+}
+
+extern "C" int vtdge_compress(const void *x, const int64_t *patches, const int64_t *rows_dev, int64_t rows,
+                              void *out, void *ln_out, const void *ln_weight, const void *ln_bias, float ln_eps,
+                              int B, int N, int C, int W, int extra, int dtype, void *stream)
+{
+    VT_REQUIRE(x && patches && out, VTDGE_ERR_ARG, "compress: NULL operand");
+    VT_REQUIRE(B > 0 && N > 0 && W > 0 && extra >= 0 && rows >= 0, VTDGE_ERR_ARG, "compress: bad sizes");
+    VT_REQUIRE((N - extra) % W == 0, VTDGE_ERR_ARG, "compress: N-extra=%d is not a multiple of W=%d", N - extra, W);
+    if (int rc = check_channels(C, dtype, "compress")) return rc;
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(C / vec <= WAVE * MAX_IT, VTDGE_ERR_UNSUPPORTED, "compress: C=%d exceeds %d", C, WAVE * MAX_IT * vec);
+    VT_REQUIRE(aligned16(x) && aligned16(out), VTDGE_ERR_ARG, "compress: operands must be 16-byte aligned");
+    const bool ln = ln_out != nullptr;
+    VT_REQUIRE(!ln || (ln_weight && ln_bias && aligned16(ln_out)), VTDGE_ERR_ARG,
+               "compress: fused LayerNorm needs weight and bias");
+    if (rows == 0) return VTDGE_OK;
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+#define VT_LAUNCH(T, LNF)                                                                                          \
+    compress_kernel<T, LNF><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out, (T *)ln_out,  \
+                                                    (const T *)ln_weight, (const T *)ln_bias, ln_eps, N, C, W, extra)
+    if (dtype == VTDGE_F32) {
+        if (ln) VT_LAUNCH(float, true); else VT_LAUNCH(float, false);
+    } else {
+        if (ln) VT_LAUNCH(bf16_t, true); else VT_LAUNCH(bf16_t, false);
+    }
+#undef VT_LAUNCH
+    return check_launch("compress");
+}
+
+extern "C" int vtdge_decompress(const void *in, const void *sub, const int64_t *patches, const int64_t *rows_dev,
+                                int64_t rows, const void *ref, void *out, int B, int N, int C, int W, int extra,
+                                int dtype, void *stream)
+{
+    VT_REQUIRE(in && patches && out, VTDGE_ERR_ARG, "decompress: NULL operand");
+    VT_REQUIRE(B > 0 && N > 0 && W > 0 && extra >= 0 && rows >= 0, VTDGE_ERR_ARG, "decompress: bad sizes");
+    VT_REQUIRE((N - extra) % W == 0, VTDGE_ERR_ARG, "decompress: N-extra=%d is not a multiple of W=%d", N - extra,
+               W);
+    if (int rc = check_channels(C, dtype, "decompress")) return rc;
+    VT_REQUIRE(aligned16(in) && aligned16(out) && aligned16(sub) && aligned16(ref), VTDGE_ERR_ARG,
+               "decompress: operands must be 16-byte aligned");
+    if (rows == 0) return VTDGE_OK;
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+#define VT_LAUNCH(T, SUBF, ADDF)                                                                                 \
+    decompress_kernel<T, SUBF, ADDF><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev,   \
+                                                             rows, (const T *)ref, (T *)out, N, C, W, extra)
+#define VT_DISPATCH(T)                                       \
+    do {                                                     \
+        if (sub && ref) VT_LAUNCH(T, true, true);            \
+        else if (sub) VT_LAUNCH(T, true, false);             \
+        else if (ref) VT_LAUNCH(T, false, true);             \
+        else VT_LAUNCH(T, false, false);                     \
+    } while (0)
+    if (dtype == VTDGE_F32) VT_DISPATCH(float); else VT_DISPATCH(bf16_t);
+#undef VT_DISPATCH
+#undef VT_LAUNCH
+    return check_launch("decompress");
+}
+
+extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,
+                               const int64_t *rows_dev, int64_t rows, int C, float eps, int dtype, void *stream)
+{
+    VT_REQUIRE(x && weight && bias && out, VTDGE_ERR_ARG, "layernorm: NULL operand");
+    VT_REQUIRE(rows >= 0, VTDGE_ERR_ARG, "layernorm: negative rows");
+    if (int rc = check_channels(C, dtype, "layernorm")) return rc;
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(C / vec <= WAVE * MAX_IT, VTDGE_ERR_UNSUPPORTED, "layernorm: C=%d exceeds %d", C,
+               WAVE * MAX_IT * vec);
+    VT_REQUIRE(aligned16(x) && aligned16(out) && aligned16(weight) && aligned16(bias), VTDGE_ERR_ARG,
+               "layernorm: operands must be 16-byte aligned");
+    if (rows == 0) return VTDGE_OK;
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_F32)
+        layernorm_kernel<float><<<grid, block, 0, st>>>((const float *)x, (const float *)weight, (const float *)bias,
+                                                        (float *)out, rows_dev, rows, C, eps);
+    else
+        layernorm_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t *)x, (const bf16_t *)weight,
+                                                         (const bf16_t *)bias, (bf16_t *)out, rows_dev, rows, C, eps);
+    return check_launch("layernorm");
+}

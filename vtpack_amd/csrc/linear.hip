@@ -1,0 +1,212 @@
+// Packed-M Linear for gfx950: out = act(A W^T + bias) + residual on MFMA.
+//
+// Both operands are K-contiguous (A [M,K], W [N,K]), which is exactly what the
+// gfx950 MFMA wants: every lane feeds 16 bytes of one operand row per
+// instruction group.  In bytes the two precisions share one geometry: a 32-byte
+// K-slab of a row is consumed by
+//   bf16: one  v_mfma_f32_32x32x16_bf16 (lane group g holds elements 8g..8g+7)
+//   fp32: four v_mfma_f32_32x32x2_f32   (lane group g holds floats 4g..4g+3;
+//         instruction j takes float j of both groups -- the contraction index
+//         is merely permuted identically for both operands)
+// so one kernel template serves both.
+//
+// Tiling: 128x128 output tile per 256-thread workgroup (2x2 waves of 64x64,
+// each 2x2 MFMA blocks of 32x32), K advanced 128 bytes per step through a
+// double-buffered LDS stage (row pitch 144 B: the 16-byte pad makes the
+// 16-lane phases of ds_read_b128 conflict free).  Workgroups are renumbered so
+// that the eight XCDs (round-robin over consecutive workgroup ids) each walk a
+// contiguous range of tiles and the N-tiles that share an A tile meet in one L2.
+#include "common.h"
+
+namespace vtdge {
+
+constexpr int BM = 128, BN = 128;
+constexpr int KB = 128;               // K bytes per stage
+constexpr int PITCH = KB + 16;        // LDS row pitch in bytes
+constexpr int NXCD = 8;
+
+__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f)); }
+
+template <typename T, int ACT, bool HAS_BIAS, bool HAS_RES>
+__global__ __launch_bounds__(256) void linear_kernel(const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt,
+                                                      const T *__restrict__ bias, const T *__restrict__ res,
+                                                      int64_t ldr, T *__restrict__ out, int64_t ldo,
+                                                      const int64_t *__restrict__ rows_dev, int64_t rows, int N,
+                                                      int K)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int ESZ = sizeof(T);
+    constexpr int STAGE = (BM + BN) * PITCH;
+
+    const int64_t M = live_rows(rows_dev, rows);
+    const int tiles_n = (N + BN - 1) / BN;
+    const int64_t tiles_m = (M + BM - 1) / BM;
+    const int64_t total = tiles_m * tiles_n;
+    const int64_t per_xcd = (total + NXCD - 1) / NXCD;
+    const int64_t local = blockIdx.x / NXCD;
+    const int64_t tile = (int64_t)(blockIdx.x % NXCD) * per_xcd + local;
+    if (local >= per_xcd || tile >= total) return;
+    const int64_t m0 = (tile / tiles_n) * BM;
+    const int n0 = (int)(tile % tiles_n) * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wid = tid >> 6;
+    const int wm = wid >> 1, wn = wid & 1;
+    const int lr = lane & 31, lg = lane >> 5;
+
+    const int64_t kbytes = (int64_t)K * ESZ;
+    const int nk = (int)((kbytes + KB - 1) / KB);
+
+    // global -> register staging: 4 A chunks + 4 W chunks of 16 B per thread
+    u32x4 ra[4], rw[4];
+    auto load_global = [&](int kt) {
+        const int64_t kb0 = (int64_t)kt * KB;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + 256 * i;
+            const int r = idx >> 3, ch = idx & 7;
+            const int64_t kb = kb0 + ch * 16;
+            const int64_t gm = m0 + r;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            ra[i] = z;
+            rw[i] = z;
+            if (gm < M && kb < kbytes)
+                ra[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const unsigned char *>(A + gm * lda) + kb);
+            const int gn = n0 + r;
+            if (gn < N && kb < kbytes)
+                rw[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const unsigned char *>(Wt + (int64_t)gn * K) +
+                                                        kb);
+        }
+    };
+    auto store_lds = [&](int buf) {
+        unsigned char *sa = smem + buf * STAGE;
+        unsigned char *sw = sa + BM * PITCH;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + 256 * i;
+            const int r = idx >> 3, ch = idx & 7;
+            *reinterpret_cast<u32x4 *>(sa + r * PITCH + ch * 16) = ra[i];
+            *reinterpret_cast<u32x4 *>(sw + r * PITCH + ch * 16) = rw[i];
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+        if (kt + 1 < nk) load_global(kt + 1);
+        const unsigned char *sa = smem + (kt & 1) * STAGE + (wm * 64 + lr) * PITCH + lg * 16;
+        const unsigned char *sw = smem + (kt & 1) * STAGE + BM * PITCH + (wn * 64 + lr) * PITCH + lg * 16;
+#pragma unroll
+        for (int s = 0; s < KB / 32; s++) {
+            u32x4 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                fa[i] = *reinterpret_cast<const u32x4 *>(sa + i * 32 * PITCH + s * 32);
+                fb[i] = *reinterpret_cast<const u32x4 *>(sw + i * 32 * PITCH + s * 32);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) Slab<T>::mma(fa[i], fb[j], acc[i][j]);
+        }
+        if (kt + 1 < nk) store_lds((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column lr of each 32x32 block, rows 8*(v/4) + 4*lg + v%4
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int col = n0 + wn * 64 + j * 32 + lr;
+        if (col >= N) continue;
+        float bv = 0.f;
+        if constexpr (HAS_BIAS) bv = Elem<T>::load(bias + col);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
+                if (row < M) {
+                    float val = acc[i][j][v] + bv;
+                    if constexpr (ACT == VTDGE_ACT_GELU) val = gelu_erf(val);
+                    if constexpr (HAS_RES) val += Elem<T>::load(res + row * ldr + col);
+                    Elem<T>::store(out + row * ldo + col, val);
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+static int launch_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
+                         void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K, int act,
+                         hipStream_t st)
+{
+    const int64_t tiles = ceil_div(rows, BM) * ceil_div(N, BN);
+    const int64_t per_xcd = ceil_div(tiles, NXCD);
+    dim3 grid((unsigned)(per_xcd * NXCD)), block(256);
+    const size_t lds = 2 * (BM + BN) * PITCH;
+#define VT_GO(ACT, HB, HR)                                                                                      \
+    do {                                                                                                        \
+        auto kern = linear_kernel<T, ACT, HB, HR>;                                                              \
+        static bool attr_done = false; /* one flag per instantiation */                                         \
+        if (!attr_done) {                                                                                       \
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                       \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {      \
+                set_error("linear: cannot reserve %zu bytes of LDS", lds);                                      \
+                return VTDGE_ERR_LAUNCH;                                                                        \
+            }                                                                                                   \
+            attr_done = true;                                                                                   \
+        }                                                                                                       \
+        kern<<<grid, block, lds, st>>>((const T *)A, lda, (const T *)W, (const T *)bias, (const T *)res, ldr,   \
+                                       (T *)out, ldo, rows_dev, rows, N, K);                                    \
+    } while (0)
+    const bool hb = bias != nullptr, hr = res != nullptr;
+    if (act == VTDGE_ACT_GELU) {
+        if (hb && hr) VT_GO(VTDGE_ACT_GELU, true, true);
+        else if (hb) VT_GO(VTDGE_ACT_GELU, true, false);
+        else if (hr) VT_GO(VTDGE_ACT_GELU, false, true);
+        else VT_GO(VTDGE_ACT_GELU, false, false);
+    } else {
+        if (hb && hr) VT_GO(VTDGE_ACT_NONE, true, true);
+        else if (hb) VT_GO(VTDGE_ACT_NONE, true, false);
+        else if (hr) VT_GO(VTDGE_ACT_NONE, false, true);
+        else VT_GO(VTDGE_ACT_NONE, false, false);
+    }
+#undef VT_GO
+    return check_launch("linear");
+}
+
+}  // namespace vtdge
+
+using namespace vtdge;
+
+extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,
+                            int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K,
+                            int act, int dtype, void *stream)
+{
+    VT_REQUIRE(A && W && out, VTDGE_ERR_ARG, "linear: NULL operand");
+    VT_REQUIRE(dtype == VTDGE_F32 || dtype == VTDGE_BF16, VTDGE_ERR_ARG, "linear: unknown dtype %d", dtype);
+    VT_REQUIRE(act == VTDGE_ACT_NONE || act == VTDGE_ACT_GELU, VTDGE_ERR_ARG, "linear: unknown activation %d", act);
+    VT_REQUIRE(rows >= 0 && N > 0 && K > 0, VTDGE_ERR_ARG, "linear: bad sizes rows=%lld N=%d K=%d", (long long)rows,
+               N, K);
+    const int esz = dtype == VTDGE_BF16 ? 2 : 4;
+    VT_REQUIRE(((int64_t)K * esz) % 16 == 0 && (lda * esz) % 16 == 0, VTDGE_ERR_UNSUPPORTED,
+               "linear: K=%d and lda=%lld must be multiples of %d elements", K, (long long)lda, 16 / esz);
+    VT_REQUIRE(lda >= K && ldo >= N && (!residual || ldr >= N), VTDGE_ERR_ARG, "linear: leading dim too small");
+    VT_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, VTDGE_ERR_ARG,
+               "linear: A and W must be 16-byte aligned");
+    if (rows == 0) return VTDGE_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_F32)
+        return launch_linear<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
+    return launch_linear<bf16_t>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
+}

@@ -1,0 +1,109 @@
+"""DynamicGrainedEncoder / DynamicRouter on the HIP kernels (mirror of vtpack/layers/dge.py).
+
+Module, parameter and `states` key names follow the reference so that its checkpoints and the
+code that reads `states` (the transformer block, the complexity counter) keep working.  Only the
+inference branch (argmax gate, sparse compress / decompress; dge.py:74-79, :108-111) is built;
+the training branches raise.
+"""
+import math
+from typing import List
+
+import torch
+from torch import nn
+
+from .. import ops
+from .grained_sample import grained_sample_compress, grained_sample_decompress, grained_sample_index_to_patch
+
+
+class DynamicRouter(nn.Module):
+    """Region mean -> Linear(C, #splits).  vtpack/layers/dge.py:115-150."""
+
+    def __init__(self, num_channels, split_sizes, init_gate=0.95):
+        super().__init__()
+        self.num_channels = num_channels
+        self.split_sizes = list(split_sizes)
+        self.region_size = max(self.split_sizes)
+        self.init_gate = init_gate
+        self.gate = nn.Linear(num_channels, len(self.split_sizes))
+        self.init_parameters()
+
+    def init_parameters(self):
+        # dge.py:129-138: tiny weights; bias so that the finest split starts with probability init_gate
+        nn.init.trunc_normal_(self.gate.weight, std=.01)
+        n = len(self.split_sizes)
+        with torch.no_grad():
+            if n == 1:
+                self.gate.bias.zero_()
+            else:
+                b = math.log(math.sqrt(self.init_gate * (1 - n) / (self.init_gate - 1)))
+                self.gate.bias.fill_(-b)
+                self.gate.bias[0] = b
+
+    def complexity(self, num_inputs, num_queries):
+        per_region = num_inputs / (self.region_size ** 2) * self.num_channels
+        return per_region + per_region * len(self.split_sizes)
+
+    def route(self, x_tokens, H, W):
+        """x_tokens [B, extra+H*W, C] -> (gate logits [B,Hr,Wr,S], argmax indices int64 [B,Hr,Wr])."""
+        return ops.router(x_tokens, self.gate.weight, self.gate.bias, H, W, self.region_size)
+
+    def forward(self, x):
+        """x [B,H,W,C] -> gate logits [B,Hr,Wr,S] (the reference's call form, dge.py:145-150)."""
+        B, H, W, C = x.shape
+        return self.route(x.reshape(B, H * W, C), H, W)[0]
+
+
+class DynamicGrainedEncoder(nn.Module):
+
+    def __init__(self, in_channels: int, split_sizes: List[int], complexity_handler=None, sparse_train: bool = False):
+        super().__init__()
+        self.in_channels = in_channels
+        self.region_size = max(split_sizes)
+        for s in split_sizes:
+            if s <= 0 or self.region_size % s:
+                raise ValueError(f"split size {s} does not divide the region size {self.region_size}")
+        self.splits = nn.Parameter(torch.tensor(list(split_sizes), dtype=torch.int64), requires_grad=False)
+        self.router = DynamicRouter(in_channels, split_sizes)
+        self.complexity_handler = complexity_handler
+        self.sparse_train = sparse_train
+        self.states = {"comp": None, "input": None, "patches": None, "batches": None, "gate": None, "size": None,
+                       "num_extra_tokens": 0}
+
+    def get_complexity(self):
+        # vtpack/layers/dge.py:40-59
+        if self.complexity_handler is None:
+            return {"static": None, "dynamic": None}
+        B, N, _ = self.states["input"].shape
+        gate = self.states["gate"]
+        if not self.training:
+            gate = torch.zeros_like(gate).scatter_(-1, gate.argmax(dim=-1, keepdim=True), 1.0)
+        per_region = gate.double() * (self.splits.to(gate.device).double() ** 2)
+        num_queries = per_region.reshape(B, -1).sum(-1) + self.states["num_extra_tokens"]
+        num_inputs = torch.full_like(num_queries, N)
+        router_cost = self.router.complexity(num_inputs, num_queries)
+        return {"static": self.complexity_handler(num_inputs, num_inputs) + router_cost,
+                "dynamic": self.complexity_handler(num_inputs, num_queries) + router_cost}
+
+    def compress(self, x, H, W, gate=None):
+        """x [B, extra+H*W, C] -> packed queries [L, C].  `gate` overrides the router output (tests)."""
+        if self.training:
+            raise NotImplementedError("only the inference branch of the Dynamic Grained Encoder is built")
+        B, N, C = x.shape
+        extra = N - H * W
+        if gate is None:
+            gate, indices = self.router.route(x, H, W)
+        else:
+            indices = gate.argmax(dim=-1)
+        patches, batches = grained_sample_index_to_patch(indices, self.splits, self.region_size, extra)
+        comp = grained_sample_compress(x, patches, H, W, extra)
+        self.states.update({"comp": comp, "input": x, "patches": patches, "batches": batches, "gate": gate,
+                            "size": (H, W), "num_extra_tokens": extra})
+        return comp
+
+    def decompress(self, x):
+        """packed [L, C] -> tokens [B, N, C]: input + broadcast(x - comp).  dge.py:87-111."""
+        if self.training:
+            raise NotImplementedError("only the inference branch of the Dynamic Grained Encoder is built")
+        st = self.states
+        return grained_sample_decompress(x - st["comp"], st["patches"], st["input"], *st["size"],
+                                         st["num_extra_tokens"], True)

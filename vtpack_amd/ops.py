@@ -1,0 +1,137 @@
+"""Thin tensor-level wrappers over the C ABI (include/vtdge.h).
+
+Every function here only checks shapes, allocates outputs with torch and hands
+raw device pointers plus the current HIP stream to libvtdge.  Row counts of
+packed operands may stay on the device (`rows_dev`), so nothing in this module
+synchronises with the GPU.
+"""
+import torch
+
+from . import _lib
+from ._lib import call, dtype_code, ptr, stream_ptr
+
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("vtdge operators run on the GPU only (got a CPU tensor); there is no CPU fallback")
+
+
+def _contig(t):
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def router(x, weight, bias, H, W, region_size, want_gate=True):
+    """AvgPool(R) -> Linear -> argmax on the spatial tokens of x [B, extra+H*W, C].
+
+    Returns (gate [B,Hr,Wr,S] or None, indices int64 [B,Hr,Wr]).  vtpack/layers/dge.py:145-150, :75.
+    """
+    _need_gpu(x, weight, bias)
+    x, weight, bias = _contig(x), _contig(weight), _contig(bias)
+    B, N, C = x.shape
+    S = weight.shape[0]
+    extra = N - H * W
+    Hr, Wr = H // region_size, W // region_size
+    gate = torch.empty((B, Hr, Wr, S), dtype=x.dtype, device=x.device) if want_gate else None
+    indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
+    weight, bias = weight.to(x.dtype), bias.to(x.dtype)
+    call("vtdge_router", ptr(x), ptr(weight), ptr(bias), ptr(gate), ptr(indices), B, H, W, C,
+         extra, region_size, S, dtype_code(x), stream_ptr())
+    return gate, indices
+
+
+def index_to_patch(indices, splits, region_size, num_extra_tokens, capacity=None):
+    """Device-only compaction: (patches [capacity,4], offsets [B+1], lengths [B]), all on the GPU."""
+    _need_gpu(indices, splits)
+    indices, splits = _contig(indices), _contig(splits)
+    B, Hr, Wr = indices.shape
+    if capacity is None:
+        capacity = B * (num_extra_tokens + Hr * Wr * region_size * region_size)
+    patches = torch.empty((capacity, 4), dtype=torch.int64, device=indices.device)
+    offsets = torch.empty((B + 1,), dtype=torch.int64, device=indices.device)
+    lengths = torch.empty((B,), dtype=torch.int64, device=indices.device)
+    call("vtdge_index_to_patch", ptr(indices), ptr(splits), B, Hr, Wr, splits.numel(), region_size,
+         num_extra_tokens, ptr(patches), capacity, ptr(offsets), ptr(lengths), stream_ptr())
+    return patches, offsets, lengths
+
+
+def compress(x, patches, width, num_extra_tokens, rows_dev=None, rows=None, ln_weight=None, ln_bias=None,
+             ln_eps=1e-6):
+    """x [B,N,C] -> comp [rows,C] (and LayerNorm(comp) when ln_weight is given)."""
+    _need_gpu(x, patches)
+    x, patches = _contig(x), _contig(patches)
+    B, N, C = x.shape
+    rows = patches.shape[0] if rows is None else rows
+    out = torch.empty((rows, C), dtype=x.dtype, device=x.device)
+    ln_out = torch.empty_like(out) if ln_weight is not None else None
+    call("vtdge_compress", ptr(x), ptr(patches), ptr(rows_dev), rows, ptr(out), ptr(ln_out), ptr(ln_weight),
+         ptr(ln_bias), float(ln_eps), B, N, C, width, num_extra_tokens, dtype_code(x), stream_ptr())
+    return (out, ln_out) if ln_weight is not None else out
+
+
+def decompress(inp, patches, reference, width, num_extra_tokens, add_ref=True, sub=None, rows_dev=None, rows=None,
+               out=None):
+    """Scatter (inp - sub) back over the tokens each patch covers, plus reference when add_ref."""
+    _need_gpu(inp, patches, reference, sub)
+    inp, patches, reference = _contig(inp), _contig(patches), _contig(reference)
+    sub = None if sub is None else _contig(sub)
+    B, N, C = reference.shape
+    rows = patches.shape[0] if rows is None else rows
+    if out is None:
+        out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
+    call("vtdge_decompress", ptr(inp), ptr(sub), ptr(patches), ptr(rows_dev), rows,
+         ptr(reference) if add_ref else 0, ptr(out), B, N, C, width, num_extra_tokens, dtype_code(inp), stream_ptr())
+    return out
+
+
+def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
+    _need_gpu(x, weight, bias)
+    x = _contig(x)
+    C = x.shape[-1]
+    rows = x.numel() // C
+    if out is None:
+        out = torch.empty_like(x)
+    call("vtdge_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(rows_dev), rows, C, float(eps),
+         dtype_code(x), stream_ptr())
+    return out
+
+
+def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=None):
+    """out = act(a @ weight.T + bias) + residual; a [..., K] (last dim contiguous), weight [N, K]."""
+    _need_gpu(a, weight, bias, residual)
+    K = a.shape[-1]
+    a2 = a.reshape(-1, K)
+    if a2.stride(-1) != 1:
+        a2 = a2.contiguous()
+    weight = _contig(weight)
+    N = weight.shape[0]
+    rows = a2.shape[0]
+    if out is None:
+        out = torch.empty(a.shape[:-1] + (N,), dtype=a.dtype, device=a.device)
+    o2 = out.view(-1, N)
+    r2 = None
+    if residual is not None:
+        r2 = residual.reshape(-1, N)
+        if r2.stride(-1) != 1:
+            r2 = r2.contiguous()
+    call("vtdge_linear", ptr(a2), a2.stride(0) if rows > 1 else K, ptr(weight), ptr(bias), ptr(r2),
+         (r2.stride(0) if rows > 1 else N) if r2 is not None else 0, ptr(o2), o2.stride(0) if rows > 1 else N,
+         ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr())
+    return out
+
+
+def sparse_attention(q, k, v, offsets, scale, num_heads, max_rows_per_sample, out=None):
+    """Strided form.  q [L, h*d]; k, v [B, n, h*d]-like views (last dim contiguous, any batch/token strides);
+    offsets int64 [B+1] on the device.  Returns [L, h*d] with channel = head*d + j."""
+    _need_gpu(q, k, v, offsets)
+    L, C = q.shape
+    d = C // num_heads
+    B, n = k.shape[0], k.shape[1]
+    assert k.stride(-1) == 1 and v.stride(-1) == 1 and q.stride(-1) == 1
+    assert k.stride() == v.stride()
+    if out is None:
+        out = torch.empty((L, C), dtype=q.dtype, device=q.device)
+    call("vtdge_sparse_attention", ptr(q), q.stride(0), d, ptr(k), ptr(v), k.stride(0), k.stride(1), d,
+         ptr(offsets), ptr(out), out.stride(0), d, B, num_heads, d, n, int(max_rows_per_sample), float(scale),
+         dtype_code(q), stream_ptr())
+    return out
