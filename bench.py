@@ -1,0 +1,284 @@
+#!/usr/bin/env python3
+"""Benchmark of the DGE query path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg4] [--no-graph]
+
+A step is one inference forward of DeiT+DGE over one batch of synthetic images already resident in HBM.
+The headline workload is BASELINE.json's configs[2] ("cfg3": DeiT-S+DGE, 12 layers, bf16, 256 px, batch 256,
+router set for a ~0.5 complexity ratio).  One JSON line is printed:
+
+  value         images/s over the K timed steps (wall clock between two device synchronisations)
+  roofline      the kernel name with the largest share of GPU time: algorithmic flops (or bytes) of its launches
+                divided by their HIP-event durations, against MI355X's published peak
+  kernels       the same figures for every libvtdge kernel of the step
+  cpu_baseline  the torch-CPU restatement of the same model (oracle/torch_ref.py) timed on this box's host cores
+                on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"hbm": 8000.0,                         # GB/s
+        "mfma": {"bf16": 2500.0, "f32": 157.3}}  # TFLOP/s, dense
+
+WORKLOADS = {
+    # name: (factory, img, batch, dtype, heads, description)
+    "cfg2": ("deit_dge_s124_tiny_patch16_256", 256, 128, "f32", 3, "DeiT-Ti+DGE 12L fp32 256px B128"),
+    "cfg3": ("deit_dge_s124_small_patch16_256", 256, 256, "bf16", 6, "DeiT-S+DGE 12L bf16 256px B256"),
+    "cfg5": ("deit_dge_s124_small_patch16_256", 512, 64, "bf16", 6, "DeiT-S+DGE 12L bf16 512px B64"),
+}
+
+
+class EventTimer:
+    """Brackets every libvtdge call with a pair of HIP events on the stream the kernels are launched on."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.records = []
+        self._open = None
+
+    def begin(self, name, tag):
+        s = self.torch.cuda.Event(enable_timing=True)
+        e = self.torch.cuda.Event(enable_timing=True)
+        s.record()
+        self._open = (name, tag, s, e)
+
+    def end(self):
+        name, tag, s, e = self._open
+        e.record()
+        self.records.append((name, tag, s, e))
+
+    def durations(self):
+        self.torch.cuda.synchronize()
+        return [(n, t, s.elapsed_time(e) * 1e-3) for n, t, s, e in self.records]
+
+
+def kernel_symbol(name, tag, dt):
+    """Name under which rocprofv3 lists the kernel a call launches (T = float or unsigned short)."""
+    T = "unsigned short" if dt == "bf16" else "float"
+    b = lambda v: "true" if v else "false"  # noqa: E731
+    if name == "vtdge_linear":
+        act = 1 if tag[1] == "gelu" else 0
+        return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
+    if name == "vtdge_compress":
+        return f"compress_kernel<{T}, {b(tag[1])}>"
+    if name == "vtdge_decompress":
+        return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}>"
+    if name == "vtdge_layernorm":
+        return f"layernorm_kernel<{T}>"
+    if name == "vtdge_sparse_attention":
+        return f"sparse_attention_kernel<{T}, {tag[3]}>"
+    if name == "vtdge_router":
+        return f"router_kernel<{T}>"
+    if name == "vtdge_index_to_patch":
+        return "patch_count_scan_kernel+patch_write_kernel"
+    return name
+
+
+def algorithmic_work(name, tag, esz, geo):
+    """(bound, amount) per launch: flops for MFMA kernels, bytes for HBM kernels.
+
+    geo: dict with B, N, C, L (live packed rows of the layer the launch belongs to), regions."""
+    B, N, C, L = geo["B"], geo["N"], geo["C"], geo["L"]
+    if name == "vtdge_linear":
+        _, _, _, _, rows, Nn, K, packed = tag
+        M = L if packed else rows
+        return "mfma", 2.0 * M * Nn * K
+    if name == "vtdge_sparse_attention":
+        return "mfma", 4.0 * L * N * C
+    if name == "vtdge_compress":
+        # read every token once, the descriptors, write every query once (+ the fused LayerNorm copy)
+        return "hbm", B * N * C * esz + 32 * L + L * C * esz * (2 if tag[1] else 1)
+    if name == "vtdge_decompress":
+        return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + (2 if tag[2] else 1) * B * N * C * esz
+    if name == "vtdge_layernorm":
+        rows = L if tag[1] else geo["ln_rows"]
+        return "hbm", 2.0 * rows * C * esz
+    if name == "vtdge_router":
+        return "hbm", B * (N - geo["extra"]) * C * esz
+    if name == "vtdge_index_to_patch":
+        return "hbm", 8.0 * B * geo["regions"] + 32 * L + 8 * B
+    return "hbm", 0.0
+
+
+def run_model_workload(args, torch):
+    from vtpack_amd import _lib
+    from vtpack_amd.models import dge as zoo
+    from vtpack_amd.synthetic import set_synthetic_router, synthetic_images
+
+    factory, img, batch, dt, heads, desc = WORKLOADS[args.workload]
+    if args.batch:
+        batch = args.batch
+    dtype = torch.bfloat16 if dt == "bf16" else torch.float32
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    model = getattr(zoo, factory)(img_size=img)
+    set_synthetic_router(model, 0)
+    model = model.eval().to(dev).to(dtype)
+    images = synthetic_images(batch, img, seed=0, dtype=dtype, device=dev)
+
+    def step():
+        with torch.no_grad():
+            return model(images)
+
+    for _ in range(max(args.warmup, 1)):
+        out = step()
+    torch.cuda.synchronize()
+
+    # ---- optional HIP graph of the whole forward, validated against the eager result on several replays
+    mode = "eager"
+    runner = step
+    if not args.no_graph:
+        try:
+            static_out = None
+            g = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            with torch.cuda.graph(g):
+                static_out = step()
+            ok = True
+            for _ in range(3):
+                eager = step()
+                torch.cuda.synchronize()
+                g.replay()
+                torch.cuda.synchronize()
+                ok = ok and torch.equal(static_out, eager)
+            if ok:
+                mode = "hipgraph"
+                runner = g.replay
+            else:
+                print("bench: graph replay differs from the eager result; timing the eager path", file=sys.stderr)
+        except Exception as exc:  # capture is an optimisation, never a requirement
+            print(f"bench: HIP graph capture unavailable ({exc}); timing the eager path", file=sys.stderr)
+            torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        runner()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        runner()
+    torch.cuda.synchronize()
+    dt_s = time.perf_counter() - t0
+    ms_per_step = dt_s / args.steps * 1e3
+    value = batch * args.steps / dt_s
+
+    # ---- per-kernel HIP-event timing: the same steps again, eagerly, every libvtdge launch bracketed
+    timer = EventTimer(torch)
+    inst_steps = min(args.steps, 5)
+    lens = []
+    _lib.timer = timer
+    try:
+        for _ in range(inst_steps):
+            step()
+            lens.append([int(b.dge.states["offsets_device"][-1]) for b in model.blocks])
+    finally:
+        _lib.timer = None
+    recs = timer.durations()
+
+    N = model.pos_embed.shape[1]
+    C = model.embed_dim
+    esz = 2 if dt == "bf16" else 4
+    G = img // 16
+    per_step = len(recs) // inst_steps
+    per_block = (per_step - 3) // len(model.blocks)   # patch embed + blocks + final norm + head
+    stats = {}
+    for i, (name, tag, sec) in enumerate(recs):
+        j = i % per_step
+        # launches of one step: 1 patch-embed linear, per_block per block, then final norm + head
+        layer = min(max((j - 1) // per_block, 0), len(model.blocks) - 1)
+        L = lens[i // per_step][layer]
+        geo = {"B": batch, "N": N, "C": C, "L": L, "regions": (G // 4) ** 2, "extra": 1, "ln_rows": batch * N}
+        if name == "vtdge_layernorm" and j == per_step - 2:
+            geo["ln_rows"] = batch
+        bound, amount = algorithmic_work(name, tag, esz, geo)
+        sym = kernel_symbol(name, tag, dt)
+        st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0})
+        st["launches"] += 1
+        st["seconds"] += sec
+        st["work"] += amount
+    kernels = {}
+    for sym, st in stats.items():
+        peak = PEAK["hbm"] if st["bound"] == "hbm" else PEAK["mfma"][dt]
+        unit = "GB/s" if st["bound"] == "hbm" else "TFLOP/s"
+        ach = st["work"] / st["seconds"] / (1e9 if st["bound"] == "hbm" else 1e12)
+        kernels[sym] = {"bound": st["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
+                        "frac": round(ach / peak, 4), "avg_us": round(st["seconds"] / st["launches"] * 1e6, 2),
+                        "launches_per_step": st["launches"] // inst_steps,
+                        "share": 0.0}
+    tot = sum(st["seconds"] for st in stats.values())
+    for sym, st in stats.items():
+        kernels[sym]["share"] = round(st["seconds"] / tot, 4)
+    dom = max(stats, key=lambda s: stats[s]["seconds"])
+    roof = {k: kernels[dom][k] for k in ("bound", "achieved", "peak", "unit", "frac")}
+    roof.update({"kernel": dom, "avg_us": kernels[dom]["avg_us"], "traffic": None})
+
+    ratio = sum(sum(l) for l in lens) / (len(lens) * len(model.blocks) * batch * N)
+    result = {
+        "metric": "images/sec DeiT-S+DGE bf16 256px @1 MI355X" if args.workload == "cfg3"
+        else f"images/sec {desc} @1 MI355X",
+        "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {desc}, budget~0.5 via synthetic router", "batch": batch,
+                   "tokens": N, "query_ratio": round(ratio, 4), "mode": mode},
+        "roofline": roof, "kernels": kernels,
+    }
+    return result, model, images, heads
+
+
+def cpu_baseline(args, torch, model, images, heads):
+    """The torch-CPU restatement on a bounded sample of the same workload, on this box's host cores."""
+    from oracle import torch_ref
+    sample = min(args.cpu_sample, images.shape[0])
+    sd = torch_ref.float_state_dict(model)
+    img = images[:sample].float().cpu()
+    depth = len(model.blocks)
+    threads = torch.get_num_threads()
+    with torch.no_grad():
+        torch_ref.deit_dge_forward(sd, img, heads, depth)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            torch_ref.deit_dge_forward(sd, img, heads, depth)
+            times.append(time.perf_counter() - t0)
+    med = sorted(times)[1]
+    return {"value": round(sample / med, 2), "unit": "images/s", "cores": threads, "kind": "port",
+            "sample": f"{sample} images of the same workload, fp32 torch-CPU restatement (oracle/torch_ref.py), "
+                      f"median of 3 after 1 warm-up, {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size")
+    ap.add_argument("--no-graph", action="store_true", help="time the eager path instead of a HIP graph replay")
+    ap.add_argument("--cpu-sample", type=int, default=32, help="images in the CPU baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (the path shards along the batch with no exchange step; "
+              "see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    result, model, images, heads = run_model_workload(args, torch)
+    if args.cpu_sample > 0:
+        result["cpu_baseline"] = cpu_baseline(args, torch, model, images, heads)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -76,9 +76,17 @@ def load():
     return lib
 
 
-def call(name, *args):
+# Optional per-launch timer (benchmarks only): an object with begin(name, tag) / end(); None = off.
+timer = None
+
+
+def call(name, *args, tag=None):
     lib = load()
+    if timer is not None:
+        timer.begin(name, tag)
     rc = getattr(lib, name)(*args)
+    if timer is not None:
+        timer.end()
     if rc != 0:
         msg = lib.vtdge_last_error().decode("utf-8", "replace")
         raise VtdgeError(f"{name} failed ({rc}): {msg}")

@@ -50,3 +50,31 @@ def block_forward(block, x, H, W, gate=None):
                        "offsets_device": offsets, "gate": gate, "size": (H, W), "num_extra_tokens": extra,
                        "queries": q2})
     return out
+
+
+def model_forward(model, images):
+    """images [B, 3, S, S] -> logits for a `VisionTransformer` in eval mode, dense pieces included.
+
+    The patch embedding (a stride-16 16x16 convolution, i.e. a Linear over unfolded patches), the final
+    LayerNorm (only the class-token rows are needed) and the classifier run on the same libvtdge kernels;
+    torch contributes only the unfold / concat / add copy kernels.  vtpack/models/dge/deit_dge.py:267-299.
+    """
+    pe = model.patch_embed
+    B, Cin, S, _ = images.shape
+    if tuple(images.shape[-2:]) != pe.img_size:
+        raise ValueError(f"input {tuple(images.shape[-2:])} does not match the model's image size {pe.img_size}")
+    P = pe.patch_size[0]
+    G = S // P
+    C = model.embed_dim
+    patches = images.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
+    x = torch.empty((B, 1 + G * G, C), dtype=images.dtype, device=images.device)
+    tok = ops.linear(patches, pe.proj.weight.reshape(C, Cin * P * P), pe.proj.bias)
+    x[:, 1:, :] = tok.view(B, G * G, C)
+    x[:, :1, :] = model.cls_token
+    x += model.pos_embed
+    for blk in model.blocks:
+        x = block_forward(blk, x, G, G)
+    cls = ops.layernorm(x[:, 0, :], model.norm.weight, model.norm.bias, model.norm.eps)
+    if isinstance(model.head, torch.nn.Linear):
+        return ops.linear(cls, model.head.weight, model.head.bias)
+    return cls

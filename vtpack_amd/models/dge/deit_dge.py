@@ -130,6 +130,7 @@ class VisionTransformer(nn.Module):
             for _ in range(depth)])
         self.norm = norm_layer(embed_dim)
         self.head = nn.Linear(embed_dim, num_classes) if num_classes > 0 else nn.Identity()
+        self.fused = fused
         self._init_weights()
 
     def _init_weights(self):
@@ -149,6 +150,7 @@ class VisionTransformer(nn.Module):
                 m.router.init_parameters()
 
     def set_fused(self, fused):
+        self.fused = fused
         for blk in self.blocks:
             blk.fused = fused
         return self
@@ -168,6 +170,8 @@ class VisionTransformer(nn.Module):
         return self.norm(x)[:, 0]
 
     def forward(self, x):
+        if self.fused and not self.training:
+            return engine.model_forward(self, x)
         return self.head(self.forward_features(x))
 
 

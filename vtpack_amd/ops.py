@@ -36,7 +36,7 @@ def router(x, weight, bias, H, W, region_size, want_gate=True):
     indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
     weight, bias = weight.to(x.dtype), bias.to(x.dtype)
     call("vtdge_router", ptr(x), ptr(weight), ptr(bias), ptr(gate), ptr(indices), B, H, W, C,
-         extra, region_size, S, dtype_code(x), stream_ptr())
+         extra, region_size, S, dtype_code(x), stream_ptr(), tag=("router",))
     return gate, indices
 
 
@@ -51,7 +51,7 @@ def index_to_patch(indices, splits, region_size, num_extra_tokens, capacity=None
     offsets = torch.empty((B + 1,), dtype=torch.int64, device=indices.device)
     lengths = torch.empty((B,), dtype=torch.int64, device=indices.device)
     call("vtdge_index_to_patch", ptr(indices), ptr(splits), B, Hr, Wr, splits.numel(), region_size,
-         num_extra_tokens, ptr(patches), capacity, ptr(offsets), ptr(lengths), stream_ptr())
+         num_extra_tokens, ptr(patches), capacity, ptr(offsets), ptr(lengths), stream_ptr(), tag=("index_to_patch",))
     return patches, offsets, lengths
 
 
@@ -65,7 +65,8 @@ def compress(x, patches, width, num_extra_tokens, rows_dev=None, rows=None, ln_w
     out = torch.empty((rows, C), dtype=x.dtype, device=x.device)
     ln_out = torch.empty_like(out) if ln_weight is not None else None
     call("vtdge_compress", ptr(x), ptr(patches), ptr(rows_dev), rows, ptr(out), ptr(ln_out), ptr(ln_weight),
-         ptr(ln_bias), float(ln_eps), B, N, C, width, num_extra_tokens, dtype_code(x), stream_ptr())
+         ptr(ln_bias), float(ln_eps), B, N, C, width, num_extra_tokens, dtype_code(x), stream_ptr(),
+         tag=("compress", ln_weight is not None))
     return (out, ln_out) if ln_weight is not None else out
 
 
@@ -80,7 +81,8 @@ def decompress(inp, patches, reference, width, num_extra_tokens, add_ref=True, s
     if out is None:
         out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
     call("vtdge_decompress", ptr(inp), ptr(sub), ptr(patches), ptr(rows_dev), rows,
-         ptr(reference) if add_ref else 0, ptr(out), B, N, C, width, num_extra_tokens, dtype_code(inp), stream_ptr())
+         ptr(reference) if add_ref else 0, ptr(out), B, N, C, width, num_extra_tokens, dtype_code(inp), stream_ptr(),
+         tag=("decompress", sub is not None, bool(add_ref)))
     return out
 
 
@@ -92,7 +94,7 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     if out is None:
         out = torch.empty_like(x)
     call("vtdge_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(rows_dev), rows, C, float(eps),
-         dtype_code(x), stream_ptr())
+         dtype_code(x), stream_ptr(), tag=("layernorm", rows_dev is not None))
     return out
 
 
@@ -116,7 +118,8 @@ def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=N
             r2 = r2.contiguous()
     call("vtdge_linear", ptr(a2), a2.stride(0) if rows > 1 else K, ptr(weight), ptr(bias), ptr(r2),
          (r2.stride(0) if rows > 1 else N) if r2 is not None else 0, ptr(o2), o2.stride(0) if rows > 1 else N,
-         ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr())
+         ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr(),
+         tag=("linear", act, bias is not None, residual is not None, rows, N, K, rows_dev is not None))
     return out
 
 
@@ -133,5 +136,5 @@ def sparse_attention(q, k, v, offsets, scale, num_heads, max_rows_per_sample, ou
         out = torch.empty((L, C), dtype=q.dtype, device=q.device)
     call("vtdge_sparse_attention", ptr(q), q.stride(0), d, ptr(k), ptr(v), k.stride(0), k.stride(1), d,
          ptr(offsets), ptr(out), out.stride(0), d, B, num_heads, d, n, int(max_rows_per_sample), float(scale),
-         dtype_code(q), stream_ptr())
+         dtype_code(q), stream_ptr(), tag=("attention", B, num_heads, d, n))
     return out
