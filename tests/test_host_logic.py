@@ -1,0 +1,105 @@
+"""Host-side logic of the package: API surface, state-dict names, error behaviour, complexity counter."""
+import math
+
+import pytest
+import torch
+
+
+def test_layer_api_surface():
+    import vtpack_amd.layers as L
+    for name in ["DynamicGrainedEncoder", "grained_sample_compress", "grained_sample_decompress",
+                 "grained_sample_index_to_patch", "batched_sparse_gemm", "batched_sparse_attention"]:
+        assert hasattr(L, name)          # vtpack/layers/__init__.py:1-10
+    from vtpack_amd import _C
+    for name in ["grained_sample_compress", "grained_sample_decompress", "grained_sample_index_to_patch",
+                 "grained_sample_index_to_patch_dense", "batched_sparse_gemm_forward",
+                 "batched_sparse_gemm_v2_forward", "batched_sparse_attention_forward"]:
+        assert callable(getattr(_C, name))   # vtpack/layers/csrc/vision.cpp:11-21
+
+
+def test_install_as_vtpack_registers_operator_module():
+    import sys
+    import vtpack_amd
+    saved = {k: sys.modules.get(k) for k in ("vtpack", "vtpack._C")}
+    try:
+        c = vtpack_amd.install_as_vtpack()
+        from vtpack import _C
+        assert _C is c and callable(_C.grained_sample_compress)
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
+def test_state_dict_keys_follow_the_reference():
+    from vtpack_amd.models.dge import deit_dge_s124_tiny_patch16_256
+    m = deit_dge_s124_tiny_patch16_256()
+    keys = set(m.state_dict().keys())
+    want = {"cls_token", "pos_embed", "patch_embed.proj.weight", "patch_embed.proj.bias", "norm.weight",
+            "norm.bias", "head.weight", "head.bias"}
+    for i in range(12):
+        for k in ["norm1.weight", "norm1.bias", "attn.q.weight", "attn.q.bias", "attn.kv.weight", "attn.kv.bias",
+                  "attn.proj.weight", "attn.proj.bias", "norm2.weight", "norm2.bias", "mlp.fc1.weight",
+                  "mlp.fc1.bias", "mlp.fc2.weight", "mlp.fc2.bias", "dge.splits", "dge.router.gate.weight",
+                  "dge.router.gate.bias"]:
+            want.add(f"blocks.{i}.{k}")
+    assert keys == want
+    assert m.blocks[0].dge.splits.dtype == torch.int64 and m.blocks[0].dge.splits.tolist() == [4, 2, 1]
+    assert m.bfloat16().blocks[0].dge.splits.dtype == torch.int64      # integer data survives dtype casts
+    assert m.pos_embed.shape == (1, 257, 192) and m.blocks[0].norm1.eps == 1e-6
+
+
+def test_router_initialisation():
+    # vtpack/layers/dge.py:129-138: bias = +-1/2 ln 38 in favour of the finest split
+    from vtpack_amd.layers import DynamicGrainedEncoder
+    d = DynamicGrainedEncoder(64, [4, 2, 1])
+    b = 0.5 * math.log(38.0)
+    assert torch.allclose(d.router.gate.bias, torch.tensor([b, -b, -b]), atol=1e-6)
+    assert 0.005 < float(d.router.gate.weight.std()) < 0.015 and d.region_size == 4
+    assert torch.allclose(DynamicGrainedEncoder(64, [1]).router.gate.bias, torch.zeros(1))
+
+
+def test_operators_refuse_cpu_tensors_and_training():
+    from vtpack_amd import _C
+    from vtpack_amd.layers import DynamicGrainedEncoder
+    x = torch.zeros(1, 17, 8)
+    patches = torch.zeros(2, 4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        _C.grained_sample_compress(x, patches, 4, 4, 1)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        _C.batched_sparse_attention_forward(torch.zeros(1, 2, 64), torch.zeros(1, 1, 3, 64), torch.zeros(1, 1, 3, 64),
+                                            torch.tensor([2]), 1.0)
+    with pytest.raises(ValueError):
+        DynamicGrainedEncoder(8, [4, 3])           # 3 does not divide the region size 4
+    d = DynamicGrainedEncoder(8, [4, 2, 1]).train()
+    with pytest.raises(NotImplementedError):
+        d.compress(x, 4, 4)
+    with pytest.raises(TypeError):
+        _C.grained_sample_index_to_patch(torch.zeros(1, 1, 1, dtype=torch.int32), torch.tensor([4, 2, 1]), 4, 1)
+
+
+def _fake_states(model, gate_index):
+    B, N, C = 2, 257, model.embed_dim
+    for blk in model.blocks:
+        gate = torch.zeros(B, 4, 4, 3)
+        gate[..., gate_index] = 1.0
+        blk.dge.states.update({"input": torch.zeros(B, N, C), "gate": gate, "num_extra_tokens": 1})
+
+
+@pytest.mark.parametrize("factory,macs", [("deit_dge_s124_small_patch16_256", 6.1e9),
+                                          ("deit_dge_s124_tiny_patch16_256", 1.7e9)])
+def test_complexity_counter_reproduces_published_macs(factory, macs):
+    """Static MACs of DeiT-S / DeiT-Ti at 256 px: 6.1 G / 1.7 G (README.md:59,61 of the reference)."""
+    from vtpack_amd.models import dge as zoo
+    m = getattr(zoo, factory)().eval()
+    img = torch.zeros(2, 3, 256, 256)
+    _fake_states(m, 0)                       # all-fine gate: every token is its own query
+    c = m.complexity(img)
+    assert abs(float(c["static"]) - macs) / macs < 0.03
+    assert float(c["dynamic"]) == pytest.approx(float(c["static"]))
+    _fake_states(m, 2)                       # all-coarse gate: 17 queries per image
+    c2 = m.complexity(img)
+    assert float(c2["static"]) == pytest.approx(float(c["static"]))
+    assert 0.1 < float(c2["dynamic"]) / float(c2["static"]) < 0.4
