@@ -10,7 +10,7 @@ import subprocess
 import torch  # noqa: F401  (loaded first so that libvtdge binds to the HIP runtime torch already holds)
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libvtdge.so")
+LIB_PATH = os.environ.get("VTDGE_LIB", os.path.join(_PKG, "libvtdge.so"))   # override: kernel experiments only
 CSRC = os.path.join(_PKG, "csrc")
 
 F32, BF16 = 0, 1

@@ -185,6 +185,14 @@ static int launch_linear(const void *A, int64_t lda, const void *W, const void *
     return check_launch("linear");
 }
 
+// pipelined direct-to-LDS variant (linear_dma.hip)
+bool linear_dma_applicable(int64_t lda, int64_t ldr, int64_t ldo, int N, int K, int esz, const void *bias,
+                           const void *res, const void *out);
+template <typename T>
+int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
+                      void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K, int act,
+                      hipStream_t st);
+
 }  // namespace vtdge
 
 using namespace vtdge;
@@ -206,6 +214,11 @@ extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const voi
                "linear: A and W must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (linear_dma_applicable(lda, ldr, ldo, N, K, esz, bias, residual, out)) {
+        if (dtype == VTDGE_F32)
+            return launch_linear_dma<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
+        return launch_linear_dma<bf16_t>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
+    }
     if (dtype == VTDGE_F32)
         return launch_linear<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
     return launch_linear<bf16_t>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
