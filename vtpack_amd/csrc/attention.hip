@@ -248,6 +248,11 @@ static int launch_attention(const void *q, int64_t q_rs, int64_t q_hs, const voi
     return check_launch("sparse_attention");
 }
 
+// bf16 / head_dim 64 fast path (attention_dma.hip)
+int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const void *k, const void *v, int64_t kv_bs,
+                              int64_t kv_ts, int64_t kv_hs, const int64_t *offsets, void *out, int64_t o_rs,
+                              int64_t o_hs, int B, int h, int n, int max_rows, float scale, hipStream_t st);
+
 }  // namespace vtdge
 
 using namespace vtdge;
@@ -273,6 +278,10 @@ extern "C" int vtdge_sparse_attention(const void *q, int64_t q_row_stride, int64
                "sparse_attention: operands must be 16-byte aligned");
     if (max_rows_per_sample == 0) return VTDGE_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_BF16 && d == 64 && scale > 0.f && (int64_t)n * kv_tok_stride * 2 < (1LL << 31))
+        return launch_attention_bf16_d64(q, q_row_stride, q_head_stride, k, v, kv_batch_stride, kv_tok_stride,
+                                         kv_head_stride, offsets, out, o_row_stride, o_head_stride, B, h, n,
+                                         max_rows_per_sample, scale, st);
 #define VT_ATT(T, D)                                                                                                 \
     return launch_attention<T, D>(q, q_row_stride, q_head_stride, k, v, kv_batch_stride, kv_tok_stride,             \
                                   kv_head_stride, offsets, out, o_row_stride, o_head_stride, B, h, n,               \

@@ -114,6 +114,26 @@ template <> struct Slab<float> {
     }
 };
 
+// ---------------------------------------------------------------- direct loads to LDS
+// global_load_lds_dwordx4: every lane names 16 bytes of global memory; the wave's 1 KB lands at the wave-uniform
+// LDS address `lptr` + lane*16 without passing through VGPRs.  Completion is tracked by vmcnt.
+#define VT_GLOBAL_TO_LDS(gptr, lptr)                                                                     \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr),             \
+                                     (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding)
+template <int N> __device__ __forceinline__ void wait_vmcnt()
+{
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+__device__ __forceinline__ void block_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // ---------------------------------------------------------------- wave ops
 __device__ __forceinline__ float wave_sum(float v)
 {

@@ -26,23 +26,6 @@ namespace vtdge {
 
 constexpr int DKB = 128;  // K bytes per stage
 
-#define VT_GLOBAL_TO_LDS(gptr, lptr)                                                                     \
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gptr),             \
-                                     (__attribute__((address_space(3))) void *)(lptr), 16, 0, 0)
-
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding)
-template <int N> __device__ __forceinline__ void wait_vmcnt()
-{
-    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
-__device__ __forceinline__ void block_barrier()
-{
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 // GELU(x) = x * Phi(x).  fp32 keeps the exact erf form.  For bf16 outputs Phi is a degree-15 odd minimax
 // polynomial on [-4, 4] (x clamped there): no transcendental, 11 VALU instructions; |error| <= 1.3e-4 for
 // |x| <= 4 and <= 5.3e-5 * |x| beyond, i.e. below 1/30 of a bf16 rounding step of the result.
