@@ -82,9 +82,10 @@ __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, co
 }
 
 // ------------------------------------------------------------ index->patch
-// Step 1 (single workgroup): per-sample query counts and their exclusive scan.
-// Counts: one wave per sample, lanes over regions, wave reduction.
-// Scan: 1024 samples per pass, wave-level shuffles + LDS for the wave totals.
+// Step 1 (single workgroup): per-sample query counts and their exclusive scan, 1024 samples per pass.
+// Counts: every thread reads gate indices with independent, coalesced loads and adds the query count of its
+// region to its sample's LDS counter (integer atomics: order does not matter).
+// Scan: wave-level shuffles + LDS for the wave totals.
 __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *__restrict__ indices,
                                                                  const int64_t *__restrict__ splits, int B,
                                                                  int nreg, int S, int extra,
@@ -94,28 +95,26 @@ __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *_
     __shared__ int64_t wave_tot[16];
     __shared__ int64_t carry_s;
     __shared__ int sq[VTDGE_MAX_SPLITS];
+    __shared__ int cnt_s[1024];
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     if (threadIdx.x < VTDGE_MAX_SPLITS) {
         int ps = threadIdx.x < S ? (int)splits[threadIdx.x] : 0;
         sq[threadIdx.x] = ps * ps;
     }
     if (threadIdx.x == 0) carry_s = 0;
-    __syncthreads();
-    for (int b = wid; b < B; b += 16) {
-        int cnt = 0;
-        for (int r = lane; r < nreg; r += WAVE) {
-            int64_t g = indices[(int64_t)b * nreg + r];
-            g = g < 0 ? 0 : (g >= S ? S - 1 : g);
-            cnt += sq[g];
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, WAVE);
-        if (lane == 0) lengths[b] = (int64_t)cnt + extra;
-    }
-    __syncthreads();  // lengths[] written by this block are visible to it
     for (int base = 0; base < B; base += 1024) {
+        cnt_s[threadIdx.x] = 0;
+        __syncthreads();
+        const int nb = min(1024, B - base);
+        for (int64_t i = threadIdx.x; i < (int64_t)nb * nreg; i += 1024) {
+            int64_t g = indices[(int64_t)base * nreg + i];
+            g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+            atomicAdd(&cnt_s[i / nreg], sq[g]);
+        }
+        __syncthreads();
         const int b = base + threadIdx.x;
-        int64_t v = b < B ? lengths[b] : 0;
+        const int64_t v = b < B ? (int64_t)cnt_s[threadIdx.x] + extra : 0;
+        if (b < B) lengths[b] = v;
         int64_t inc = v;
 #pragma unroll
         for (int o = 1; o < WAVE; o <<= 1) {
