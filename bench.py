@@ -58,12 +58,19 @@ class EventTimer:
         return [(n, t, s.elapsed_time(e) * 1e-3) for n, t, s, e in self.records]
 
 
-def kernel_symbol(name, tag, dt):
-    """Name under which rocprofv3 lists the kernel a call launches (T = float or unsigned short)."""
+def kernel_symbol(name, tag, dt, n_keys=0):
+    """Name under which rocprofv3 lists the kernel a call launches (T = float or unsigned short).
+
+    Mirrors the host-side dispatch of libvtdge for the shapes of these workloads (all operands 16-byte aligned)."""
     T = "unsigned short" if dt == "bf16" else "float"
+    esz = 2 if dt == "bf16" else 4
     b = lambda v: "true" if v else "false"  # noqa: E731
     if name == "vtdge_linear":
         act = 1 if tag[1] == "gelu" else 0
+        N, K = tag[5], tag[6]
+        if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
+            tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
+            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     if name == "vtdge_compress":
         return f"compress_kernel<{T}, {b(tag[1])}>"
@@ -72,12 +79,28 @@ def kernel_symbol(name, tag, dt):
     if name == "vtdge_layernorm":
         return f"layernorm_kernel<{T}>"
     if name == "vtdge_sparse_attention":
+        if dt == "bf16" and tag[3] == 64:
+            return "sparse_attention_bf16_d64_resident_kernel" if tag[4] <= 288 else "sparse_attention_bf16_d64_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
         return f"router_kernel<{T}>"
     if name == "vtdge_index_to_patch":
         return "patch_count_scan_kernel+patch_write_kernel"
     return name
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch by kernel name, from the committed rocprofv3 --pmc summary of this workload
+    (FETCH_SIZE / WRITE_SIZE scaled by a copy of known size); {} when there is none."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}_pmc.txt")
+    table = {}
+    if os.path.exists(path):
+        for line in open(path):
+            if line.startswith("#") or "|" not in line:
+                continue
+            cols = [c.strip() for c in line.split("|")]
+            table[cols[0]] = int(cols[4])
+    return table
 
 
 def algorithmic_work(name, tag, esz, geo):
@@ -219,7 +242,18 @@ def run_model_workload(args, torch):
         kernels[sym]["share"] = round(st["seconds"] / tot, 4)
     dom = max(stats, key=lambda s: stats[s]["seconds"])
     roof = {k: kernels[dom][k] for k in ("bound", "achieved", "peak", "unit", "frac")}
-    roof.update({"kernel": dom, "avg_us": kernels[dom]["avg_us"], "traffic": None})
+    traffic = measured_traffic(args.workload)
+    for sym in kernels:
+        kernels[sym]["algorithmic_per_launch"] = int(stats[sym]["work"] / stats[sym]["launches"])
+        kernels[sym]["traffic"] = traffic.get(sym)
+    roof.update({"kernel": dom, "avg_us": kernels[dom]["avg_us"], "traffic": traffic.get(dom)})
+
+    # one plain device-to-device copy of known size (256 MiB), so that a counter run of this script carries its
+    # own yardstick for the HBM byte counters
+    calib_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    calib_dst = torch.empty_like(calib_src)
+    calib_dst.copy_(calib_src)
+    torch.cuda.synchronize()
 
     ratio = sum(sum(l) for l in lens) / (len(lens) * len(model.blocks) * batch * N)
     result = {
@@ -233,6 +267,58 @@ def run_model_workload(args, torch):
         "roofline": roof, "kernels": kernels,
     }
     return result, model, images, heads
+
+
+def run_isolated_gemm(args, torch):
+    """cfg4: packed A [L, 384] ~ N(0,1) against shared W [N, 384] ~ N(0, 0.02), bf16; 256 segments whose lengths
+    follow a seeded skewed gate mix (1/4/16 queries per region with a heavy tail), clipped to [16, 256]."""
+    import numpy as np
+    from vtpack_amd import ops
+    dev = torch.device("cuda:0")
+    rng = np.random.RandomState(0)
+    p_fine = np.clip(rng.beta(0.6, 2.0, size=256), 0, 1)          # most samples coarse, a heavy tail of fine ones
+    lengths = []
+    for pf in p_fine:
+        probs = [pf, (1 - pf) * 0.4, (1 - pf) * 0.6]
+        lengths.append(1 + int(rng.choice([16, 4, 1], size=16, p=probs).sum()))
+    lengths = np.clip(np.array(lengths), 16, 256)
+    L = int(lengths.sum())
+    K = 384
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn((L, K), generator=g).to(dev, torch.bfloat16)
+    rows_dev = torch.tensor([L], dtype=torch.int64, device=dev)
+    per_n, total_flops, total_s = {}, 0.0, 0.0
+    for N in (384, 1152, 1536):
+        Wt = (torch.randn((N, K), generator=g) * 0.02).to(dev, torch.bfloat16)
+        bias = torch.zeros(N, device=dev, dtype=torch.bfloat16)
+        out = torch.empty((L, N), device=dev, dtype=torch.bfloat16)
+        for _ in range(args.warmup):
+            ops.linear(A, Wt, bias, rows_dev=rows_dev, out=out)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        s.record()
+        for _ in range(args.steps):
+            ops.linear(A, Wt, bias, rows_dev=rows_dev, out=out)
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / args.steps
+        fl = 2.0 * L * N * K
+        byts = (L * K + N * K + L * N) * 2
+        per_n[str(N)] = {"us": round(sec * 1e6, 2), "TFLOP/s": round(fl / sec / 1e12, 1),
+                         "GB/s": round(byts / sec / 1e9, 1), "frac_mfma": round(fl / sec / 1e12 / 2500.0, 4)}
+        total_flops += fl
+        total_s += sec
+    ach = total_flops / total_s / 1e12
+    return {"metric": "TFLOP/s isolated packed-M GEMM bf16 K=384 @1 MI355X", "value": round(ach, 1),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(total_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "cfg4: 256 segments, skewed lengths in [16,256], K=384, N in {384,1152,1536}",
+                       "packed_rows": L},
+            "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": round(ach / 2500.0, 4), "kernel": "linear_dma_kernel<unsigned short, ...>",
+                         "traffic": None},
+            "per_n": per_n}
 
 
 def cpu_baseline(args, torch, model, images, heads):
@@ -261,7 +347,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size")
     ap.add_argument("--no-graph", action="store_true", help="time the eager path instead of a HIP graph replay")
     ap.add_argument("--cpu-sample", type=int, default=32, help="images in the CPU baseline sample (0 = skip)")
@@ -274,6 +360,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "cfg4":
+        print(json.dumps(run_isolated_gemm(args, torch)))
+        return
     result, model, images, heads = run_model_workload(args, torch)
     if args.cpu_sample > 0:
         result["cpu_baseline"] = cpu_baseline(args, torch, model, images, heads)
