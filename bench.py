@@ -145,6 +145,8 @@ def run_model_workload(args, torch):
     model = model.eval().to(dev).to(dtype)
     images = synthetic_images(batch, img, seed=0, dtype=dtype, device=dev)
 
+    from vtpack_amd import engine
+
     def step():
         with torch.no_grad():
             return model(images)
@@ -199,12 +201,14 @@ def run_model_workload(args, torch):
     inst_steps = min(args.steps, 5)
     lens = []
     _lib.timer = timer
+    engine.OVERLAP = False      # one kernel at a time on one stream
     try:
         for _ in range(inst_steps):
             step()
             lens.append([int(b.dge.states["offsets_device"][-1]) for b in model.blocks])
     finally:
         _lib.timer = None
+        engine.OVERLAP = True
     recs = timer.durations()
 
     N = model.pos_embed.shape[1]

@@ -135,11 +135,20 @@ __device__ __forceinline__ void block_barrier()
 }
 
 // ---------------------------------------------------------------- wave ops
+// Sum over the 64 lanes, returned in every lane.  DPP row shifts inside rows of 16 lanes, row broadcasts
+// across rows (total in lane 63), one readlane: six short-latency VALU ops instead of six LDS permutes.
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
+#define VT_DPP_ADD(ctrl, row_mask) \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, true))
+    VT_DPP_ADD(0x111, 0xf);  // row_shr:1
+    VT_DPP_ADD(0x112, 0xf);  // row_shr:2
+    VT_DPP_ADD(0x114, 0xf);  // row_shr:4
+    VT_DPP_ADD(0x118, 0xf);  // row_shr:8
+    VT_DPP_ADD(0x142, 0xa);  // row_bcast:15
+    VT_DPP_ADD(0x143, 0xc);  // row_bcast:31
+#undef VT_DPP_ADD
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_max(float v)
 {

@@ -14,7 +14,7 @@ constexpr int MAX_IT = 3;          // 16-byte vectors per lane: C <= 64*3*VEC
 // ------------------------------------------------------------------ router
 // One wave per region.  Replaces AvgPool2d(R,R) -> Linear(C,S) -> argmax
 // (vtpack/layers/dge.py:145-150, :75).
-template <typename T>
+template <typename T, int RS>   // RS = region size known at compile time (all window loads in flight), 0 = generic
 __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, const T *__restrict__ weight,
                                                       const T *__restrict__ bias, T *__restrict__ gate,
                                                       int64_t *__restrict__ indices, int B, int H, int W,
@@ -41,14 +41,30 @@ __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, co
         float acc[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) acc[i] = 0.f;
-        for (int dy = 0; dy < R; dy++) {
-            for (int dx = 0; dx < R; dx++) {
-                const int tok = (ry * R + dy) * W + rx * R + dx + extra;
-                u32x4 raw = *reinterpret_cast<const u32x4 *>(xb + (int64_t)tok * C + v * VEC);
+        const T *base = xb + ((int64_t)(ry * R) * W + rx * R + extra) * C + v * VEC;
+        if constexpr (RS > 0) {
+            u32x4 raw[RS * RS];
+#pragma unroll
+            for (int dy = 0; dy < RS; dy++)
+#pragma unroll
+                for (int dx = 0; dx < RS; dx++)
+                    raw[dy * RS + dx] = *reinterpret_cast<const u32x4 *>(base + ((int64_t)dy * W + dx) * C);
+#pragma unroll
+            for (int t = 0; t < RS * RS; t++) {
                 float f[VEC];
-                Elem<T>::unpack(raw, f);
+                Elem<T>::unpack(raw[t], f);
 #pragma unroll
                 for (int i = 0; i < VEC; i++) acc[i] += f[i];
+            }
+        } else {
+            for (int dy = 0; dy < R; dy++) {
+                for (int dx = 0; dx < R; dx++) {
+                    u32x4 raw = *reinterpret_cast<const u32x4 *>(base + ((int64_t)dy * W + dx) * C);
+                    float f[VEC];
+                    Elem<T>::unpack(raw, f);
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) acc[i] += f[i];
+                }
             }
         }
 #pragma unroll
@@ -433,7 +449,9 @@ __global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ i
 }
 
 // --------------------------------------------------------------- layernorm
-template <typename T>
+constexpr int LN_RPW = 4;   // rows per wave: their loads are issued together so that enough bytes are in flight
+
+template <typename T, int NIT>   // NIT = 16-byte vectors per lane = ceil(C / VEC / 64)
 __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                          const T *__restrict__ bsrc, T *__restrict__ out,
                                                          const int64_t *__restrict__ rows_dev, int64_t rows, int C,
@@ -441,43 +459,63 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
 {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
-    if (row >= live_rows(rows_dev, rows)) return;
+    const int64_t live = live_rows(rows_dev, rows);
+    const int64_t row0 = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * LN_RPW;
+    if (row0 >= live) return;
     const int nvec = C / VEC;
-    float vals[MAX_IT][VEC];
-    float s = 0.f;
+    u32x4 raw[LN_RPW][NIT];
 #pragma unroll
-    for (int it = 0; it < MAX_IT; it++) {
+    for (int r = 0; r < LN_RPW; r++)
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int v = it * WAVE + lane;
+            if (v < nvec && row0 + r < live)
+                raw[r][it] = *reinterpret_cast<const u32x4 *>(x + (row0 + r) * (int64_t)C + v * VEC);
+        }
+    float ww[NIT][VEC], bb[NIT][VEC];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
         const int v = it * WAVE + lane;
         if (v < nvec) {
-            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(x + row * (int64_t)C + v * VEC), vals[it]);
-#pragma unroll
-            for (int c = 0; c < VEC; c++) s += vals[it][c];
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(w + v * VEC), ww[it]);
+            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(bsrc + v * VEC), bb[it]);
         }
     }
-    const float mean = wave_sum(s) / (float)C;
-    float q = 0.f;
 #pragma unroll
-    for (int it = 0; it < MAX_IT; it++) {
-        if (it * WAVE + lane < nvec) {
+    for (int r = 0; r < LN_RPW; r++) {
+        if (row0 + r >= live) break;
+        float vals[NIT][VEC];
+        float s = 0.f;
 #pragma unroll
-            for (int c = 0; c < VEC; c++) {
-                const float dlt = vals[it][c] - mean;
-                q += dlt * dlt;
+        for (int it = 0; it < NIT; it++) {
+            if (it * WAVE + lane < nvec) {
+                Elem<T>::unpack(raw[r][it], vals[it]);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) s += vals[it][c];
             }
         }
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+        const float mean = wave_sum(s) / (float)C;
+        float q = 0.f;
 #pragma unroll
-    for (int it = 0; it < MAX_IT; it++) {
-        const int v = it * WAVE + lane;
-        if (v < nvec) {
-            float ww[VEC], bb[VEC], y[VEC];
-            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(w + v * VEC), ww);
-            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(bsrc + v * VEC), bb);
+        for (int it = 0; it < NIT; it++) {
+            if (it * WAVE + lane < nvec) {
 #pragma unroll
-            for (int c = 0; c < VEC; c++) y[c] = (vals[it][c] - mean) * rstd * ww[c] + bb[c];
-            *reinterpret_cast<u32x4 *>(out + row * (int64_t)C + v * VEC) = Elem<T>::pack(y);
+                for (int c = 0; c < VEC; c++) {
+                    const float dlt = vals[it][c] - mean;
+                    q += dlt * dlt;
+                }
+            }
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int v = it * WAVE + lane;
+            if (v < nvec) {
+                float y[VEC];
+#pragma unroll
+                for (int c = 0; c < VEC; c++) y[c] = (vals[it][c] - mean) * rstd * ww[it][c] + bb[it][c];
+                *reinterpret_cast<u32x4 *>(out + (row0 + r) * (int64_t)C + v * VEC) = Elem<T>::pack(y);
+            }
         }
     }
 }
@@ -513,13 +551,15 @@ extern "C" int vtdge_router(const void *x, const void *weight, const void *bias,
     const int64_t regions = (int64_t)B * (H / R) * (W / R);
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == VTDGE_F32)
-        router_kernel<float><<<grid, block, 0, st>>>((const float *)x, (const float *)weight, (const float *)bias,
-                                                     (float *)gate, indices, B, H, W, C, extra, R, S);
-    else
-        router_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t *)x, (const bf16_t *)weight,
-                                                      (const bf16_t *)bias, (bf16_t *)gate, indices, B, H, W, C,
-                                                      extra, R, S);
+#define VT_LAUNCH(T, RS)                                                                                       \
+    router_kernel<T, RS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)gate, indices, \
+                                                 B, H, W, C, extra, R, S)
+    if (dtype == VTDGE_F32) {
+        if (R == 4) VT_LAUNCH(float, 4); else if (R == 2) VT_LAUNCH(float, 2); else VT_LAUNCH(float, 0);
+    } else {
+        if (R == 4) VT_LAUNCH(bf16_t, 4); else if (R == 2) VT_LAUNCH(bf16_t, 2); else VT_LAUNCH(bf16_t, 0);
+    }
+#undef VT_LAUNCH
     return check_launch("router");
 }
 
@@ -635,13 +675,17 @@ extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bi
     VT_REQUIRE(aligned16(x) && aligned16(out) && aligned16(weight) && aligned16(bias), VTDGE_ERR_ARG,
                "layernorm: operands must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
-    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * LN_RPW)), block(256);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == VTDGE_F32)
-        layernorm_kernel<float><<<grid, block, 0, st>>>((const float *)x, (const float *)weight, (const float *)bias,
-                                                        (float *)out, rows_dev, rows, C, eps);
-    else
-        layernorm_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t *)x, (const bf16_t *)weight,
-                                                         (const bf16_t *)bias, (bf16_t *)out, rows_dev, rows, C, eps);
+    const int nit = (int)ceil_div(C / vec, WAVE);
+#define VT_LAUNCH(T, NIT)                                                                                        \
+    layernorm_kernel<T, NIT><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
+                                                     rows_dev, rows, C, eps)
+    if (dtype == VTDGE_F32) {
+        if (nit == 1) VT_LAUNCH(float, 1); else if (nit == 2) VT_LAUNCH(float, 2); else VT_LAUNCH(float, 3);
+    } else {
+        if (nit == 1) VT_LAUNCH(bf16_t, 1); else if (nit == 2) VT_LAUNCH(bf16_t, 2); else VT_LAUNCH(bf16_t, 3);
+    }
+#undef VT_LAUNCH
     return check_launch("layernorm");
 }

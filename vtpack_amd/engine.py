@@ -10,11 +10,26 @@ import torch
 
 from . import ops
 
+# The block has two independent chains before attention: the routing chain (router -> index->patch -> compress ->
+# q projection: small, latency-bound launches) and the key/value chain (LayerNorm of all tokens -> kv projection:
+# the largest GEMM).  They are issued on two HIP streams of equal (default) priority and joined before attention,
+# in eager mode and inside a captured graph alike.
+_side_streams = {}
+OVERLAP = True          # module switch (benchmarks turn it off to time kernels one at a time)
 
-def block_forward(block, x, H, W, gate=None):
+
+def _side_stream(device, slot=0):
+    s = _side_streams.get((device, slot))
+    if s is None:
+        s = _side_streams[(device, slot)] = torch.cuda.Stream(device=device)
+    return s
+
+
+def block_forward(block, x, H, W, gate=None, overlap=True):
     """x [B, N, C] -> [B, N, C] for a `vtpack_amd.models.dge.deit_dge.Block` in eval mode.
 
     `gate` [B, Hr, Wr, S] overrides the router's logits (used by the parity tests).
+    `overlap` issues the key/value chain on a second stream next to the routing chain.
     """
     dge, attn, mlp = block.dge, block.attn, block.mlp
     B, N, C = x.shape
@@ -22,6 +37,19 @@ def block_forward(block, x, H, W, gate=None):
     R = dge.region_size
     x = x.contiguous()
 
+    n1, n2 = block.norm1, block.norm2
+    overlap = overlap and OVERLAP
+    main = torch.cuda.current_stream(x.device)
+    side = _side_stream(x.device, main.cuda_stream) if overlap else main
+
+    # key/value chain (second stream)
+    if overlap:
+        side.wait_stream(main)
+    with torch.cuda.stream(side):
+        x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
+        kv = ops.linear(x_ln, attn.kv.weight, attn.kv.bias)                   # [B, N, 2C] = [B, N, 2, h, d]
+
+    # routing chain (caller's stream)
     if gate is None:
         gate, indices = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
     else:
@@ -29,14 +57,14 @@ def block_forward(block, x, H, W, gate=None):
     cap = B * N
     patches, offsets, lengths = ops.index_to_patch(indices, dge.splits, R, extra, capacity=cap)
     rows_dev = offsets[B:]
-
-    n1, n2 = block.norm1, block.norm2
     comp, comp_ln = ops.compress(x, patches, W, extra, rows_dev=rows_dev, rows=cap, ln_weight=n1.weight,
                                  ln_bias=n1.bias, ln_eps=n1.eps)
-    x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
-
     q = ops.linear(comp_ln, attn.q.weight, attn.q.bias, rows_dev=rows_dev)
-    kv = ops.linear(x_ln, attn.kv.weight, attn.kv.bias)                       # [B, N, 2C] = [B, N, 2, h, d]
+
+    if overlap:
+        main.wait_stream(side)
+        for t in (x_ln, kv):
+            t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
     q1 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev)
 
