@@ -116,7 +116,8 @@ int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *o
  * [L, C] (vtpack/models/dge/deit_dge.py:72,96,38-44) and kv on [B*N, C] (:73).
  *   A [rows, K] leading dim lda      W [N, K] dense      bias [N] nullable
  *   residual [rows, N] leading dim ldr, nullable         out [rows, N] leading dim ldo
- * MFMA kernel; K must be a multiple of 32 bytes worth of elements (8 fp32 / 16 bf16). */
+ * MFMA kernels; K must be a multiple of 16 bytes worth of elements (4 fp32 / 8 bf16).  Rows of K that are a
+ * multiple of 128 bytes (and 16-byte aligned operands) take the direct-to-LDS persistent kernel. */
 int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,
                  int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K,
                  int act, int dtype, void *stream);
