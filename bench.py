@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the DGE query path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg4] [--no-graph]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg4|pvt] [--no-graph]
 
 A step is one inference forward of DeiT+DGE over one batch of synthetic images already resident in HBM.
 The headline workload is BASELINE.json's configs[2] ("cfg3": DeiT-S+DGE, 12 layers, bf16, 256 px, batch 256,
@@ -31,6 +31,8 @@ WORKLOADS = {
     "cfg2": ("deit_dge_s124_tiny_patch16_256", 256, 128, "f32", 3, "DeiT-Ti+DGE 12L fp32 256px B128"),
     "cfg3": ("deit_dge_s124_small_patch16_256", 256, 256, "bf16", 6, "DeiT-S+DGE 12L bf16 256px B256"),
     "cfg5": ("deit_dge_s124_small_patch16_256", 512, 64, "bf16", 6, "DeiT-S+DGE 12L bf16 512px B64"),
+    # the second caller of the path (PVT: four stages, spatially reduced keys/values); not a BASELINE config
+    "pvt": ("pvt_dge_s124_small_256", 256, 256, "bf16", (1, 2, 5, 8), "PVT-S+DGE 16L bf16 256px B256"),
 }
 
 
@@ -106,22 +108,22 @@ def measured_traffic(workload):
 def algorithmic_work(name, tag, esz, geo):
     """(bound, amount) per launch: flops for MFMA kernels, bytes for HBM kernels.
 
-    geo: dict with B, N, C, L (live packed rows of the layer the launch belongs to), regions."""
+    geo: dict with B, N, C, L (live packed rows), regions and extra of the block the launch belongs to."""
     B, N, C, L = geo["B"], geo["N"], geo["C"], geo["L"]
     if name == "vtdge_linear":
         _, _, _, _, rows, Nn, K, packed = tag
         M = L if packed else rows
         return "mfma", 2.0 * M * Nn * K
     if name == "vtdge_sparse_attention":
-        return "mfma", 4.0 * L * N * C
+        return "mfma", 4.0 * L * tag[4] * C               # tag[4] = keys per sample
     if name == "vtdge_compress":
         # read every token once, the descriptors, write every query once (+ the fused LayerNorm copy)
         return "hbm", B * N * C * esz + 32 * L + L * C * esz * (2 if tag[1] else 1)
     if name == "vtdge_decompress":
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + (2 if tag[2] else 1) * B * N * C * esz
     if name == "vtdge_layernorm":
-        rows = L if tag[1] else geo["ln_rows"]
-        return "hbm", 2.0 * rows * C * esz
+        rows = L if tag[1] else tag[2]
+        return "hbm", 2.0 * rows * tag[3] * esz
     if name == "vtdge_router":
         return "hbm", B * (N - geo["extra"]) * C * esz
     if name == "vtdge_index_to_patch":
@@ -142,6 +144,8 @@ def run_model_workload(args, torch):
     torch.manual_seed(0)
     model = getattr(zoo, factory)(img_size=img)
     set_synthetic_router(model, 0)
+    blocks = list(model.blocks) if hasattr(model, "blocks") else \
+        [b for i in range(model.num_stages) for b in getattr(model, f"block{i + 1}")]
     model = model.eval().to(dev).to(dtype)
     images = synthetic_images(batch, img, seed=0, dtype=dtype, device=dev)
 
@@ -205,33 +209,36 @@ def run_model_workload(args, torch):
     try:
         for _ in range(inst_steps):
             step()
-            lens.append([int(b.dge.states["offsets_device"][-1]) for b in model.blocks])
+            lens.append([int(b.dge.states["offsets_device"][-1]) for b in blocks])
     finally:
         _lib.timer = None
         engine.OVERLAP = True
     recs = timer.durations()
 
-    N = model.pos_embed.shape[1]
-    C = model.embed_dim
+    # geometry of every block (token count, width, regions), from the states its encoder keeps
     esz = 2 if dt == "bf16" else 4
-    G = img // 16
+    geos = []
+    for b in blocks:
+        st_ = b.dge.states
+        Bn, Nn, Cn = st_["input"].shape
+        H_, W_ = st_["size"]
+        geos.append({"B": Bn, "N": Nn, "C": Cn, "regions": (H_ // 4) * (W_ // 4), "extra": st_["num_extra_tokens"]})
     per_step = len(recs) // inst_steps
-    per_block = (per_step - 3) // len(model.blocks)   # patch embed + blocks + final norm + head
     stats = {}
+    blk = 0
     for i, (name, tag, sec) in enumerate(recs):
-        j = i % per_step
-        # launches of one step: 1 patch-embed linear, per_block per block, then final norm + head
-        layer = min(max((j - 1) // per_block, 0), len(model.blocks) - 1)
-        L = lens[i // per_step][layer]
-        geo = {"B": batch, "N": N, "C": C, "L": L, "regions": (G // 4) ** 2, "extra": 1, "ln_rows": batch * N}
-        if name == "vtdge_layernorm" and j == per_step - 2:
-            geo["ln_rows"] = batch
+        if i % per_step == 0:
+            blk = 0
+        # a block's launches end with its scatter; what precedes block 0 or follows the last block is dense
+        geo = dict(geos[min(blk, len(blocks) - 1)], L=lens[i // per_step][min(blk, len(blocks) - 1)])
         bound, amount = algorithmic_work(name, tag, esz, geo)
         sym = kernel_symbol(name, tag, dt)
         st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0})
         st["launches"] += 1
         st["seconds"] += sec
         st["work"] += amount
+        if name == "vtdge_decompress":
+            blk += 1
     kernels = {}
     for sym, st in stats.items():
         peak = PEAK["hbm"] if st["bound"] == "hbm" else PEAK["mfma"][dt]
@@ -259,7 +266,8 @@ def run_model_workload(args, torch):
     calib_dst.copy_(calib_src)
     torch.cuda.synchronize()
 
-    ratio = sum(sum(l) for l in lens) / (len(lens) * len(model.blocks) * batch * N)
+    ratio = sum(sum(l) for l in lens) / (len(lens) * sum(g["B"] * g["N"] for g in geos))
+    N = geos[-1]["N"]
     result = {
         "metric": "images/sec DeiT-S+DGE bf16 256px @1 MI355X" if args.workload == "cfg3"
         else f"images/sec {desc} @1 MI355X",
@@ -331,14 +339,19 @@ def cpu_baseline(args, torch, model, images, heads):
     sample = min(args.cpu_sample, images.shape[0])
     sd = torch_ref.float_state_dict(model)
     img = images[:sample].float().cpu()
-    depth = len(model.blocks)
     threads = torch.get_num_threads()
+    if hasattr(model, "blocks"):
+        depth = len(model.blocks)
+        run = lambda: torch_ref.deit_dge_forward(sd, img, heads, depth)  # noqa: E731
+    else:
+        sr = [getattr(model, f"block{i + 1}")[0].attn.sr_ratio for i in range(model.num_stages)]
+        run = lambda: torch_ref.pvt_dge_forward(sd, img, heads, model.depths, sr)  # noqa: E731
     with torch.no_grad():
-        torch_ref.deit_dge_forward(sd, img, heads, depth)
+        run()
         times = []
         for _ in range(3):
             t0 = time.perf_counter()
-            torch_ref.deit_dge_forward(sd, img, heads, depth)
+            run()
             times.append(time.perf_counter() - t0)
     med = sorted(times)[1]
     return {"value": round(sample / med, 2), "unit": "images/s", "cores": threads, "kind": "port",

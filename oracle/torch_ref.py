@@ -117,16 +117,21 @@ def sparse_gemm(a, b, a_lengths, b_lengths, ta, tb):
 
 
 # ----------------------------------------------------------------------------- block / model
-def block_forward(sd, prefix, x, num_heads, gate=None, indices=None, eps=1e-6, trace=None):
-    """vtpack/models/dge/deit_dge.py:123-130 (eval) for the block whose keys start with `prefix`.
+def block_forward(sd, prefix, x, num_heads, gate=None, indices=None, eps=1e-6, trace=None, size=None, sr_ratio=1,
+                  sr_eps=1e-5):
+    """vtpack/models/dge/deit_dge.py:123-130 and vtpack/models/dge/pvt_dge.py:134-140 (eval) for the block whose
+    keys start with `prefix`.
 
     gate: optional logits injected in place of the router output.
     indices: optional gate indices forced on the block (teacher forcing), overriding both.
     trace: optional dict that receives every intermediate.
+    size: (H, W) of the token grid (default: square, as deit_dge.py:125 assumes).
+    sr_ratio: spatial reduction of the key/value tokens (pvt_dge.py:83-87): Conv2d(C, C, sr, stride sr) on the
+        normalised token grid, then LayerNorm(eps = sr_eps, nn.LayerNorm's default).
     """
     p = lambda name: sd[prefix + name]  # noqa: E731
     B, N, C = x.shape
-    H = W = int(math.sqrt(N))
+    H, W = size if size is not None else (int(math.sqrt(N)),) * 2
     extra = N - H * W
     splits = p("dge.splits").to(torch.int64)
     R = int(splits.max())
@@ -140,8 +145,14 @@ def block_forward(sd, prefix, x, num_heads, gate=None, indices=None, eps=1e-6, t
     ln = lambda t, n: F.layer_norm(t, (C,), p(n + ".weight"), p(n + ".bias"), eps)  # noqa: E731
     d = C // num_heads
     q = F.linear(ln(comp, "norm1"), p("attn.q.weight"), p("attn.q.bias")).reshape(-1, num_heads, d).permute(1, 0, 2)
-    kv = F.linear(ln(x, "norm1"), p("attn.kv.weight"), p("attn.kv.bias"))
-    kv = kv.reshape(B, N, 2, num_heads, d).permute(2, 3, 0, 1, 4)
+    kv_src = ln(x, "norm1")
+    if sr_ratio > 1:
+        grid = kv_src.permute(0, 2, 1).reshape(B, C, H, W)
+        grid = F.conv2d(grid, p("attn.sr.weight"), p("attn.sr.bias"), stride=sr_ratio)
+        kv_src = F.layer_norm(grid.reshape(B, C, -1).permute(0, 2, 1), (C,), p("attn.norm.weight"),
+                              p("attn.norm.bias"), sr_eps)
+    kv = F.linear(kv_src, p("attn.kv.weight"), p("attn.kv.bias"))
+    kv = kv.reshape(B, -1, 2, num_heads, d).permute(2, 3, 0, 1, 4)
     att = attention(q, kv[0], kv[1], lengths, d ** -0.5).transpose(0, 1).reshape(-1, C)
     q1 = comp + F.linear(att, p("attn.proj.weight"), p("attn.proj.bias"))
     hid = F.gelu(F.linear(ln(q1, "norm2"), p("mlp.fc1.weight"), p("mlp.fc1.bias")))
@@ -164,6 +175,41 @@ def deit_dge_forward(sd, images, num_heads, depth, patch=16, eps=1e-6, forced_in
                           indices=None if forced_indices is None else forced_indices[i])
         if traces is not None:
             traces.append(tr)
+    C = x.shape[-1]
+    x = F.layer_norm(x, (C,), sd["norm.weight"], sd["norm.bias"], eps)[:, 0]
+    return F.linear(x, sd["head.weight"], sd["head.bias"])
+
+
+def pvt_dge_forward(sd, images, num_heads, depths, sr_ratios, patch=4, eps=1e-6, embed_eps=1e-5, forced_indices=None,
+                    traces=None):
+    """vtpack/models/dge/pvt_dge.py:290-339 with a classifier.  images [B,3,S,S] -> logits.
+
+    The positional embeddings must match the token grids (no interpolation branch).  forced_indices / traces are
+    flat lists over all blocks in execution order.
+    """
+    B = images.shape[0]
+    x = images
+    nblk = 0
+    last = len(depths) - 1
+    for i, depth in enumerate(depths):
+        pre = f"patch_embed{i + 1}."
+        x = F.conv2d(x, sd[pre + "proj.weight"], sd[pre + "proj.bias"], stride=patch if i == 0 else 2)
+        H, W = x.shape[2], x.shape[3]
+        C = x.shape[1]
+        x = F.layer_norm(x.flatten(2).transpose(1, 2), (C,), sd[pre + "norm.weight"], sd[pre + "norm.bias"], embed_eps)
+        if i == last:
+            x = torch.cat((sd["cls_token"].expand(B, -1, -1), x), dim=1)
+        x = x + sd[f"pos_embed{i + 1}"]
+        for j in range(depth):
+            tr = {} if traces is not None else None
+            x = block_forward(sd, f"block{i + 1}.{j}.", x, num_heads[i], eps=eps, trace=tr, size=(H, W),
+                              sr_ratio=sr_ratios[i],
+                              indices=None if forced_indices is None else forced_indices[nblk])
+            nblk += 1
+            if traces is not None:
+                traces.append(tr)
+        if i != last:
+            x = x.reshape(B, H, W, C).permute(0, 3, 1, 2)
     C = x.shape[-1]
     x = F.layer_norm(x, (C,), sd["norm.weight"], sd["norm.bias"], eps)[:, 0]
     return F.linear(x, sd["head.weight"], sd["head.bias"])

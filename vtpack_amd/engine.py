@@ -25,8 +25,42 @@ def _side_stream(device, slot=0):
     return s
 
 
+def _khwc_weight(conv):
+    """Conv2d weight [O, C, kh, kw] as a Linear weight over channels-last patches: [O, kh*kw*C]."""
+    w = conv.weight
+    key = (w.data_ptr(), w._version, w.dtype, w.device)
+    cached = getattr(conv, "_vtdge_khwc", None)
+    if cached is None or cached[0] != key:
+        flat = w.detach().permute(0, 2, 3, 1).reshape(w.shape[0], -1).contiguous()
+        conv._vtdge_khwc = cached = (key, flat)
+    return cached[1]
+
+
+def tokens_to_patches(x, H, W, k):
+    """Channels-last tokens [B, H*W, C] -> non-overlapping k x k patches [B*(H/k)*(W/k), k*k*C] (one copy)."""
+    B, _, C = x.shape
+    return x.reshape(B, H // k, k, W // k, k, C).permute(0, 1, 3, 2, 4, 5).reshape(B * (H // k) * (W // k), k * k * C)
+
+
+def _key_value_source(attn, x_ln, H, W, extra):
+    """Tokens the keys and values are projected from: LN1(x) itself, or, with spatial reduction
+    (vtpack/models/dge/pvt_dge.py:83-87), LayerNorm(Conv2d(C, C, sr, stride sr)(LN1(x))) with the convolution run
+    as a Linear over channels-last patches."""
+    sr = getattr(attn, "sr_ratio", 1)
+    if sr <= 1:
+        return x_ln
+    if extra:
+        raise ValueError("spatial reduction needs a token grid without extra tokens")
+    if H % sr or W % sr:
+        raise ValueError(f"token grid {H}x{W} is not a multiple of the reduction ratio {sr}")
+    B, _, C = x_ln.shape
+    red = ops.linear(tokens_to_patches(x_ln, H, W, sr), _khwc_weight(attn.sr), attn.sr.bias)
+    return ops.layernorm(red, attn.norm.weight, attn.norm.bias, attn.norm.eps).view(B, -1, C)
+
+
 def block_forward(block, x, H, W, gate=None, overlap=True):
-    """x [B, N, C] -> [B, N, C] for a `vtpack_amd.models.dge.deit_dge.Block` in eval mode.
+    """x [B, N, C] -> [B, N, C] for a DGE transformer block (`models.dge.deit_dge.Block` or
+    `models.dge.pvt_dge.Block`) in eval mode.
 
     `gate` [B, Hr, Wr, S] overrides the router's logits (used by the parity tests).
     `overlap` issues the key/value chain on a second stream next to the routing chain.
@@ -47,7 +81,8 @@ def block_forward(block, x, H, W, gate=None, overlap=True):
         side.wait_stream(main)
     with torch.cuda.stream(side):
         x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
-        kv = ops.linear(x_ln, attn.kv.weight, attn.kv.bias)                   # [B, N, 2C] = [B, N, 2, h, d]
+        kv_src = _key_value_source(attn, x_ln, H, W, extra)
+        kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)                 # [B, n, 2C] = [B, n, 2, h, d]
 
     # routing chain (caller's stream)
     if gate is None:
@@ -63,7 +98,7 @@ def block_forward(block, x, H, W, gate=None, overlap=True):
 
     if overlap:
         main.wait_stream(side)
-        for t in (x_ln, kv):
+        for t in (x_ln, kv_src, kv):
             t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
     q1 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev)
@@ -106,3 +141,51 @@ def model_forward(model, images):
     if isinstance(model.head, torch.nn.Linear):
         return ops.linear(cls, model.head.weight, model.head.bias)
     return cls
+
+
+def pvt_forward(model, images):
+    """images [B, 3, S, S] -> logits (or the per-stage feature maps when the model has no classifier) for a
+    `models.dge.pvt_dge.PyramidVisionTransformer` in eval mode.  vtpack/models/dge/pvt_dge.py:295-339.
+
+    Tokens stay channels-last between stages: every stage's patch embedding (a stride-k k x k convolution) runs as
+    a Linear over k x k patches gathered from the previous stage's token grid, followed by its LayerNorm.
+    """
+    B, Cin, Hi, Wi = images.shape
+    x = None
+    outputs = {}
+    for i in range(model.num_stages):
+        pe = getattr(model, f"patch_embed{i + 1}")
+        pos = getattr(model, f"pos_embed{i + 1}")
+        k = pe.patch_size[0]
+        if i == 0:
+            H, W = Hi // k, Wi // k
+            pat = images[:, :, :H * k, :W * k].reshape(B, Cin, H, k, W, k).permute(0, 2, 4, 1, 3, 5)
+            tok = ops.linear(pat.reshape(B * H * W, Cin * k * k), pe.proj.weight.reshape(pe.proj.weight.shape[0], -1),
+                             pe.proj.bias)
+        else:
+            if H % k or W % k:
+                raise ValueError(f"token grid {H}x{W} is not a multiple of the stage's patch size {k}")
+            tok = ops.linear(tokens_to_patches(x, H, W, k), _khwc_weight(pe.proj), pe.proj.bias)
+            H, W = H // k, W // k
+        C = tok.shape[-1]
+        tok = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps).view(B, H * W, C)
+        last = i == model.num_stages - 1
+        if last:
+            x = torch.empty((B, 1 + H * W, C), dtype=tok.dtype, device=tok.device)
+            x[:, 1:, :] = tok
+            x[:, :1, :] = model.cls_token
+            if H * W != pe.num_patches:
+                pos = torch.cat((pos[:, :1], model._get_pos_embed(pos[:, 1:], pe, H, W)), dim=1)
+            x += pos
+        else:
+            x = tok + model._get_pos_embed(pos, pe, H, W)
+        for blk in getattr(model, f"block{i + 1}"):
+            x = block_forward(blk, x, H, W)
+        if not last:
+            outputs[f"res{i + 2}"] = x.view(B, H, W, C)
+        elif model.num_classes == 0:
+            outputs[f"res{i + 2}"] = x[:, 1:].reshape(B, H, W, C)
+    if model.num_classes == 0:
+        return {name: t.permute(0, 3, 1, 2).contiguous() for name, t in outputs.items()}
+    cls = ops.layernorm(x[:, 0, :], model.norm.weight, model.norm.bias, model.norm.eps)
+    return ops.linear(cls, model.head.weight, model.head.bias)

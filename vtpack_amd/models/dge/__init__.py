@@ -1,1 +1,2 @@
 from .deit_dge import *  # noqa: F401,F403
+from .pvt_dge import *  # noqa: F401,F403

@@ -94,7 +94,7 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     if out is None:
         out = torch.empty_like(x)
     call("vtdge_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(rows_dev), rows, C, float(eps),
-         dtype_code(x), stream_ptr(), tag=("layernorm", rows_dev is not None))
+         dtype_code(x), stream_ptr(), tag=("layernorm", rows_dev is not None, rows, C))
     return out
 
 

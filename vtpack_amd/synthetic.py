@@ -25,8 +25,10 @@ def set_synthetic_router(model, seed=0):
     """Zero bias + seeded N(0, 1/C) weights for every block's router (mixed gate instead of all-fine)."""
     g = torch.Generator().manual_seed(seed)
     with torch.no_grad():
-        for blk in model.blocks:
-            lin = blk.dge.router.gate
+        for mod in model.modules():
+            if not hasattr(mod, "router") or not hasattr(mod, "splits"):
+                continue                       # every DynamicGrainedEncoder, in execution order
+            lin = mod.router.gate
             w = torch.randn(lin.weight.shape, generator=g) / lin.weight.shape[1] ** 0.5
             lin.weight.copy_(w.to(lin.weight.dtype))
             lin.bias.zero_()
