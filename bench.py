@@ -74,18 +74,19 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
+    gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_compress":
-        return f"compress_kernel<{T}, {b(tag[1])}>"
+        return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}>"
     if name == "vtdge_decompress":
-        return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}>"
+        return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
     if name == "vtdge_layernorm":
-        return f"layernorm_kernel<{T}>"
+        return f"layernorm_kernel<{T}, {gs(tag[3])}>"
     if name == "vtdge_sparse_attention":
         if dt == "bf16" and tag[3] == 64:
             return "sparse_attention_bf16_d64_resident_kernel" if tag[4] <= 288 else "sparse_attention_bf16_d64_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
-        return f"router_kernel<{T}>"
+        return f"router_kernel<{T}, {gs(tag[1])}>"
     if name == "vtdge_index_to_patch":
         return "patch_count_scan_kernel+patch_write_kernel"
     return name

@@ -1,29 +1,46 @@
 // Grained sampling kernels for gfx950: router, index->patch compaction,
 // compress (gather + window mean) and decompress (scatter back).
 //
-// All four are HBM-bandwidth or latency bound.  The element kernels give one
-// 64-lane wavefront to one packed query row and move 16 bytes per lane, so a
-// row of C channels is read/written with fully coalesced 16-byte accesses.
+// All four are HBM-bandwidth or latency bound.  The element kernels give a
+// group of GS lanes (64, 32, 16 or 8: the smallest that covers C with 16 bytes
+// per lane) to one packed query row, so a row of C channels is read/written
+// with fully coalesced 16-byte accesses and narrow rows (C = 64, 128: the
+// first PVT stages) still keep every lane of the wavefront busy.
 #include "common.h"
 
 namespace vtdge {
 
-constexpr int ROWS_PER_BLOCK = 4;  // one wave per row, 256 threads
+constexpr int ROWS_PER_BLOCK = 4;  // one wave per row (GS = 64) or 64/GS rows per wave, 256 threads
 constexpr int MAX_IT = 3;          // 16-byte vectors per lane: C <= 64*3*VEC
+
+// lanes per row for a row of nvec 16-byte vectors
+static int group_size(int nvec) { return nvec > 32 ? 64 : nvec > 16 ? 32 : nvec > 8 ? 16 : 8; }
+
+// sum over the GS lanes of a row's group, returned in each of them
+template <int GS> __device__ __forceinline__ float group_sum(float v)
+{
+    if constexpr (GS == 64) {
+        return wave_sum(v);
+    } else {
+#pragma unroll
+        for (int o = GS / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+        return v;
+    }
+}
 
 // ------------------------------------------------------------------ router
 // One wave per region.  Replaces AvgPool2d(R,R) -> Linear(C,S) -> argmax
 // (vtpack/layers/dge.py:145-150, :75).
-template <typename T, int RS>   // RS = region size known at compile time (all window loads in flight), 0 = generic
+template <typename T, int RS, int GS>   // RS = region size known at compile time (all window loads in flight), 0 = generic
 __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, const T *__restrict__ weight,
                                                       const T *__restrict__ bias, T *__restrict__ gate,
                                                       int64_t *__restrict__ indices, int B, int H, int W,
                                                       int C, int extra, int R, int S)
 {
     constexpr int VEC = Elem<T>::VEC;
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & (GS - 1);
     const int Hr = H / R, Wr = W / R;
-    const int64_t region = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    const int64_t region = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
     if (region >= (int64_t)B * Hr * Wr) return;
     const int b = (int)(region / (Hr * Wr));
     const int rr = (int)(region % (Hr * Wr));
@@ -37,7 +54,7 @@ __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, co
 #pragma unroll
     for (int s = 0; s < VTDGE_MAX_SPLITS; s++) part[s] = 0.f;
 
-    for (int v = lane; v < nvec; v += WAVE) {
+    for (int v = lane; v < nvec; v += GS) {
         float acc[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) acc[i] = 0.f;
@@ -85,7 +102,7 @@ __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, co
 #pragma unroll
     for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
         if (s < S) {
-            float logit = wave_sum(part[s]) + Elem<T>::load(bias + s);
+            float logit = group_sum<GS>(part[s]) + Elem<T>::load(bias + s);
             logit = Elem<T>::round(logit);
             if (gate != nullptr && lane == 0) Elem<T>::store(gate + region * S + s, logit);
             if (s == 0 || logit > best) {  // strict >: lowest index wins a tie
@@ -282,7 +299,7 @@ __device__ __forceinline__ void window_sum(const T *__restrict__ base, int W, in
     }
 }
 
-template <typename T, bool LN>
+template <typename T, bool LN, int GS>
 __global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, const int64_t *__restrict__ patches,
                                                         const int64_t *__restrict__ rows_dev, int64_t rows,
                                                         T *__restrict__ out, T *__restrict__ ln_out,
@@ -290,8 +307,9 @@ __global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, 
                                                         float eps, int N, int C, int W, int extra)
 {
     constexpr int VEC = Elem<T>::VEC;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    constexpr int NIT = GS == 64 ? MAX_IT : 1;
+    const int lane = threadIdx.x & (GS - 1);
+    const int64_t row = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
     if (row >= live_rows(rows_dev, rows)) return;
     const int64_t *p = patches + 4 * row;
     const int64_t b = p[0], y0 = p[1], x0 = p[2];
@@ -299,9 +317,9 @@ __global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, 
     const int nvec = C / VEC;
     const T *xb = x + b * (int64_t)N * C;
 
-    float vals[MAX_IT][VEC];
+    float vals[NIT][VEC];
 #pragma unroll
-    for (int it = 0; it < MAX_IT; it++) {
+    for (int it = 0; it < NIT; it++) {
         const int v = it * WAVE + lane;
         if (v < nvec) {
             float acc[VEC];
@@ -333,13 +351,13 @@ __global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, 
     if constexpr (LN) {
         float s = 0.f;
 #pragma unroll
-        for (int it = 0; it < MAX_IT; it++)
+        for (int it = 0; it < NIT; it++)
 #pragma unroll
             for (int c = 0; c < VEC; c++) s += vals[it][c];
-        const float mean = wave_sum(s) / (float)C;
+        const float mean = group_sum<GS>(s) / (float)C;
         float q = 0.f;
 #pragma unroll
-        for (int it = 0; it < MAX_IT; it++) {
+        for (int it = 0; it < NIT; it++) {
             if (it * WAVE + lane < nvec) {
 #pragma unroll
                 for (int c = 0; c < VEC; c++) {
@@ -348,9 +366,9 @@ __global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, 
                 }
             }
         }
-        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+        const float rstd = 1.0f / sqrtf(group_sum<GS>(q) / (float)C + eps);
 #pragma unroll
-        for (int it = 0; it < MAX_IT; it++) {
+        for (int it = 0; it < NIT; it++) {
             const int v = it * WAVE + lane;
             if (v < nvec) {
                 float w[VEC], bb[VEC], y[VEC];
@@ -413,7 +431,7 @@ __device__ __forceinline__ void window_store(const T *__restrict__ ref, T *__res
     }
 }
 
-template <typename T, bool SUB, bool ADD>
+template <typename T, bool SUB, bool ADD, int GS>
 __global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ in, const T *__restrict__ sub,
                                                           const int64_t *__restrict__ patches,
                                                           const int64_t *__restrict__ rows_dev, int64_t rows,
@@ -421,14 +439,14 @@ __global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ i
                                                           int C, int W, int extra)
 {
     constexpr int VEC = Elem<T>::VEC;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & (GS - 1);
+    const int64_t row = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
     if (row >= live_rows(rows_dev, rows)) return;
     const int64_t *p = patches + 4 * row;
     const int64_t b = p[0], y0 = p[1], x0 = p[2];
     const int sz = (int)p[3];
     const int nvec = C / VEC;
-    for (int v = lane; v < nvec; v += WAVE) {
+    for (int v = lane; v < nvec; v += GS) {
         float d[VEC];
         Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(in + row * (int64_t)C + v * VEC), d);
         if constexpr (SUB) {
@@ -451,16 +469,17 @@ __global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ i
 // --------------------------------------------------------------- layernorm
 constexpr int LN_RPW = 4;   // rows per wave: their loads are issued together so that enough bytes are in flight
 
-template <typename T, int NIT>   // NIT = 16-byte vectors per lane = ceil(C / VEC / 64)
+template <typename T, int NIT, int GS>   // NIT = 16-byte vectors per lane = ceil(C / VEC / 64) (1 when GS < 64)
 __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                          const T *__restrict__ bsrc, T *__restrict__ out,
                                                          const int64_t *__restrict__ rows_dev, int64_t rows, int C,
                                                          float eps)
 {
     constexpr int VEC = Elem<T>::VEC;
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & (GS - 1);
     const int64_t live = live_rows(rows_dev, rows);
-    const int64_t row0 = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * LN_RPW;
+    const int64_t row0 =
+        (((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS) * LN_RPW;
     if (row0 >= live) return;
     const int nvec = C / VEC;
     u32x4 raw[LN_RPW][NIT];
@@ -494,7 +513,7 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
                 for (int c = 0; c < VEC; c++) s += vals[it][c];
             }
         }
-        const float mean = wave_sum(s) / (float)C;
+        const float mean = group_sum<GS>(s) / (float)C;
         float q = 0.f;
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
@@ -506,7 +525,7 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
                 }
             }
         }
-        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)C + eps);
+        const float rstd = 1.0f / sqrtf(group_sum<GS>(q) / (float)C + eps);
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
             const int v = it * WAVE + lane;
@@ -549,16 +568,20 @@ extern "C" int vtdge_router(const void *x, const void *weight, const void *bias,
     if (int rc = check_channels(C, dtype, "router")) return rc;
     VT_REQUIRE(aligned16(x) && aligned16(weight), VTDGE_ERR_ARG, "router: operands must be 16-byte aligned");
     const int64_t regions = (int64_t)B * (H / R) * (W / R);
-    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
+    const int gs = group_size(C / (dtype == VTDGE_BF16 ? 8 : 4));
+    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
-#define VT_LAUNCH(T, RS)                                                                                       \
-    router_kernel<T, RS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)gate, indices, \
-                                                 B, H, W, C, extra, R, S)
-    if (dtype == VTDGE_F32) {
-        if (R == 4) VT_LAUNCH(float, 4); else if (R == 2) VT_LAUNCH(float, 2); else VT_LAUNCH(float, 0);
-    } else {
-        if (R == 4) VT_LAUNCH(bf16_t, 4); else if (R == 2) VT_LAUNCH(bf16_t, 2); else VT_LAUNCH(bf16_t, 0);
-    }
+#define VT_LAUNCH(T, RS, GS)                                                                                     \
+    router_kernel<T, RS, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)gate, \
+                                                     indices, B, H, W, C, extra, R, S)
+#define VT_REGION(T, GS) \
+    do { if (R == 4) VT_LAUNCH(T, 4, GS); else if (R == 2) VT_LAUNCH(T, 2, GS); else VT_LAUNCH(T, 0, GS); } while (0)
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_REGION(T, 64); else if (gs == 32) VT_REGION(T, 32); else if (gs == 16) VT_REGION(T, 16); \
+         else VT_REGION(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
+#undef VT_REGION
 #undef VT_LAUNCH
     return check_launch("router");
 }
@@ -619,16 +642,20 @@ extern "C" int vtdge_compress(const void *x, const int64_t *patches, const int64
     VT_REQUIRE(!ln || (ln_weight && ln_bias && aligned16(ln_out)), VTDGE_ERR_ARG,
                "compress: fused LayerNorm needs weight and bias");
     if (rows == 0) return VTDGE_OK;
-    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    const int gs = group_size(C / vec);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
-#define VT_LAUNCH(T, LNF)                                                                                          \
-    compress_kernel<T, LNF><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out, (T *)ln_out,  \
-                                                    (const T *)ln_weight, (const T *)ln_bias, ln_eps, N, C, W, extra)
-    if (dtype == VTDGE_F32) {
-        if (ln) VT_LAUNCH(float, true); else VT_LAUNCH(float, false);
-    } else {
-        if (ln) VT_LAUNCH(bf16_t, true); else VT_LAUNCH(bf16_t, false);
-    }
+#define VT_LAUNCH(T, LNF, GS)                                                                                  \
+    compress_kernel<T, LNF, GS><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out,       \
+                                                        (T *)ln_out, (const T *)ln_weight, (const T *)ln_bias, \
+                                                        ln_eps, N, C, W, extra)
+#define VT_LNF(T, GS) do { if (ln) VT_LAUNCH(T, true, GS); else VT_LAUNCH(T, false, GS); } while (0)
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_LNF(T, 64); else if (gs == 32) VT_LNF(T, 32); else if (gs == 16) VT_LNF(T, 16); \
+         else VT_LNF(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
+#undef VT_LNF
 #undef VT_LAUNCH
     return check_launch("compress");
 }
@@ -645,19 +672,27 @@ extern "C" int vtdge_decompress(const void *in, const void *sub, const int64_t *
     VT_REQUIRE(aligned16(in) && aligned16(out) && aligned16(sub) && aligned16(ref), VTDGE_ERR_ARG,
                "decompress: operands must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
-    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(256);
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(C / vec <= WAVE * MAX_IT, VTDGE_ERR_UNSUPPORTED, "decompress: C=%d exceeds %d", C,
+               WAVE * MAX_IT * vec);
+    const int gs = group_size(C / vec);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
-#define VT_LAUNCH(T, SUBF, ADDF)                                                                                 \
-    decompress_kernel<T, SUBF, ADDF><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev,   \
-                                                             rows, (const T *)ref, (T *)out, N, C, W, extra)
-#define VT_DISPATCH(T)                                       \
-    do {                                                     \
-        if (sub && ref) VT_LAUNCH(T, true, true);            \
-        else if (sub) VT_LAUNCH(T, true, false);             \
-        else if (ref) VT_LAUNCH(T, false, true);             \
-        else VT_LAUNCH(T, false, false);                     \
+#define VT_LAUNCH(T, SUBF, ADDF, GS)                                                                              \
+    decompress_kernel<T, SUBF, ADDF, GS><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev, \
+                                                                 rows, (const T *)ref, (T *)out, N, C, W, extra)
+#define VT_DISPATCH(T, GS)                                       \
+    do {                                                         \
+        if (sub && ref) VT_LAUNCH(T, true, true, GS);            \
+        else if (sub) VT_LAUNCH(T, true, false, GS);             \
+        else if (ref) VT_LAUNCH(T, false, true, GS);             \
+        else VT_LAUNCH(T, false, false, GS);                     \
     } while (0)
-    if (dtype == VTDGE_F32) VT_DISPATCH(float); else VT_DISPATCH(bf16_t);
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_DISPATCH(T, 64); else if (gs == 32) VT_DISPATCH(T, 32); else if (gs == 16) VT_DISPATCH(T, 16); \
+         else VT_DISPATCH(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
 #undef VT_DISPATCH
 #undef VT_LAUNCH
     return check_launch("decompress");
@@ -675,17 +710,20 @@ extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bi
     VT_REQUIRE(aligned16(x) && aligned16(out) && aligned16(weight) && aligned16(bias), VTDGE_ERR_ARG,
                "layernorm: operands must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
-    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * LN_RPW)), block(256);
+    const int gs = group_size(C / vec);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * LN_RPW * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
     const int nit = (int)ceil_div(C / vec, WAVE);
-#define VT_LAUNCH(T, NIT)                                                                                        \
-    layernorm_kernel<T, NIT><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
-                                                     rows_dev, rows, C, eps)
-    if (dtype == VTDGE_F32) {
-        if (nit == 1) VT_LAUNCH(float, 1); else if (nit == 2) VT_LAUNCH(float, 2); else VT_LAUNCH(float, 3);
-    } else {
-        if (nit == 1) VT_LAUNCH(bf16_t, 1); else if (nit == 2) VT_LAUNCH(bf16_t, 2); else VT_LAUNCH(bf16_t, 3);
-    }
+#define VT_LAUNCH(T, NIT, GS)                                                                                        \
+    layernorm_kernel<T, NIT, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
+                                                         rows_dev, rows, C, eps)
+#define VT_GROUP(T)                                                                                       \
+    do {                                                                                                  \
+        if (gs == 64) { if (nit == 1) VT_LAUNCH(T, 1, 64); else if (nit == 2) VT_LAUNCH(T, 2, 64); else VT_LAUNCH(T, 3, 64); } \
+        else if (gs == 32) VT_LAUNCH(T, 1, 32); else if (gs == 16) VT_LAUNCH(T, 1, 16); else VT_LAUNCH(T, 1, 8); \
+    } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
 #undef VT_LAUNCH
     return check_launch("layernorm");
 }

@@ -36,7 +36,7 @@ def router(x, weight, bias, H, W, region_size, want_gate=True):
     indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
     weight, bias = weight.to(x.dtype), bias.to(x.dtype)
     call("vtdge_router", ptr(x), ptr(weight), ptr(bias), ptr(gate), ptr(indices), B, H, W, C,
-         extra, region_size, S, dtype_code(x), stream_ptr(), tag=("router",))
+         extra, region_size, S, dtype_code(x), stream_ptr(), tag=("router", C))
     return gate, indices
 
 
@@ -66,7 +66,7 @@ def compress(x, patches, width, num_extra_tokens, rows_dev=None, rows=None, ln_w
     ln_out = torch.empty_like(out) if ln_weight is not None else None
     call("vtdge_compress", ptr(x), ptr(patches), ptr(rows_dev), rows, ptr(out), ptr(ln_out), ptr(ln_weight),
          ptr(ln_bias), float(ln_eps), B, N, C, width, num_extra_tokens, dtype_code(x), stream_ptr(),
-         tag=("compress", ln_weight is not None))
+         tag=("compress", ln_weight is not None, rows, C))
     return (out, ln_out) if ln_weight is not None else out
 
 
@@ -82,7 +82,7 @@ def decompress(inp, patches, reference, width, num_extra_tokens, add_ref=True, s
         out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
     call("vtdge_decompress", ptr(inp), ptr(sub), ptr(patches), ptr(rows_dev), rows,
          ptr(reference) if add_ref else 0, ptr(out), B, N, C, width, num_extra_tokens, dtype_code(inp), stream_ptr(),
-         tag=("decompress", sub is not None, bool(add_ref)))
+         tag=("decompress", sub is not None, bool(add_ref), C))
     return out
 
 
