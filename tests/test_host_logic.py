@@ -73,9 +73,9 @@ def test_operators_refuse_cpu_tensors_and_training():
                                             torch.tensor([2]), 1.0)
     with pytest.raises(ValueError):
         DynamicGrainedEncoder(8, [4, 3])           # 3 does not divide the region size 4
-    d = DynamicGrainedEncoder(8, [4, 2, 1]).train()
-    with pytest.raises(NotImplementedError):
-        d.compress(x, 4, 4)
+    d = DynamicGrainedEncoder(8, [4, 2, 1], sparse_train=True).train()
+    with pytest.raises(RuntimeError, match="GPU only"):
+        d.compress(x, 4, 4)                        # sparse training uses the kernels: no CPU path either
     with pytest.raises(TypeError):
         _C.grained_sample_index_to_patch(torch.zeros(1, 1, 1, dtype=torch.int32), torch.tensor([4, 2, 1]), 4, 1)
 
@@ -103,3 +103,33 @@ def test_complexity_counter_reproduces_published_macs(factory, macs):
     c2 = m.complexity(img)
     assert float(c2["static"]) == pytest.approx(float(c["static"]))
     assert 0.1 < float(c2["dynamic"]) / float(c2["static"]) < 0.4
+
+
+def test_dense_training_branch_equals_the_sparse_statement_on_cpu():
+    """Training without sparse_train is plain torch (vtpack/layers/dge.py:68-72, :91-95): with its hard one-hot
+    gate it must give what the sparse operators give for the sampled granularity, and pass gradients to the
+    input and to the router."""
+    from oracle import torch_ref
+    from vtpack_amd.layers import DynamicGrainedEncoder
+    torch.manual_seed(3)
+    B, H, W, C, extra = 2, 8, 12, 16, 1
+    d = DynamicGrainedEncoder(C, [4, 2, 1]).train()
+    with torch.no_grad():
+        d.router.gate.bias.zero_()
+        d.router.gate.weight.normal_(0, 1.0)
+    x = torch.randn(B, extra + H * W, C, requires_grad=True)
+    comp = d.compress(x, H, W)
+    assert comp.shape[0] == B * (extra + H * W + H * W // 4 + H * W // 16) and d.states["patches"] is None
+    gate = d.states["gate"]
+    assert torch.equal(gate.sum(-1), torch.ones_like(gate.sum(-1))) and set(gate.unique().tolist()) <= {0.0, 1.0}
+    out = d.decompress(torch.tanh(comp) * 2)
+    idx = gate.argmax(-1)
+    assert len(idx.unique()) > 1
+    patches, _ = torch_ref.index_to_patch(idx, d.splits, 4, extra)
+    xd = x.detach()
+    c_ref = torch_ref.compress(xd, patches, H, W, extra)
+    want = torch_ref.decompress(torch.tanh(c_ref) * 2 - c_ref, patches, xd, H, W, extra, True)
+    assert float((out - want).abs().max()) <= 1e-5
+    out.square().sum().backward()
+    assert x.grad is not None and float(x.grad.abs().max()) > 0
+    assert float(d.router.gate.weight.grad.abs().max()) > 0

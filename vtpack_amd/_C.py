@@ -47,15 +47,30 @@ def grained_sample_index_to_patch_dense(indices, split_sizes, region_size, num_e
     return patches, torch.full((B,), per, dtype=torch.int64)
 
 
+def _pad_channels(t):
+    """The kernels move 16 bytes per lane; a channel count that is not a multiple of that (the [B, N, 1] gate map
+    of sparse training, vtpack/layers/dge.py:96-106) is zero-padded here and sliced back by the caller."""
+    vec = 16 // t.element_size()
+    C = t.shape[-1]
+    if C % vec == 0:
+        return t, C
+    return torch.nn.functional.pad(t, (0, vec - C % vec)), C
+
+
 def grained_sample_compress(input, patches, height, width, num_extra_tokens):
     """input [B,N,C], patches [L,4] -> [L,C].  grained_sample.cu:198-239."""
-    return ops.compress(input, patches, int(width), int(num_extra_tokens))
+    input, C = _pad_channels(input)
+    out = ops.compress(input, patches, int(width), int(num_extra_tokens))
+    return out if out.shape[-1] == C else out[:, :C].contiguous()
 
 
 def grained_sample_decompress(input, patches, reference, height, width, num_extra_tokens, is_add_ref):
     """input [L,C], reference [B,N,C] -> [B,N,C].  grained_sample.cu:241-300."""
     _check_same_dtype(input, reference)
-    return ops.decompress(input, patches, reference, int(width), int(num_extra_tokens), add_ref=bool(is_add_ref))
+    input, C = _pad_channels(input)
+    reference, _ = _pad_channels(reference)
+    out = ops.decompress(input, patches, reference, int(width), int(num_extra_tokens), add_ref=bool(is_add_ref))
+    return out if out.shape[-1] == C else out[..., :C].contiguous()
 
 
 def _offsets_from_lengths(lengths, device):

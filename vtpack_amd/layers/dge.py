@@ -1,18 +1,23 @@
 """DynamicGrainedEncoder / DynamicRouter on the HIP kernels (mirror of vtpack/layers/dge.py).
 
 Module, parameter and `states` key names follow the reference so that its checkpoints and the
-code that reads `states` (the transformer block, the complexity counter) keep working.  Only the
-inference branch (argmax gate, sparse compress / decompress; dge.py:74-79, :108-111) is built;
-the training branches raise.
+code that reads `states` (the transformer block, the complexity counter) keep working.  The
+inference branch (argmax gate, sparse compress / decompress; dge.py:74-79, :108-111) runs on the
+HIP kernels.  The training branches (Gumbel hard gate; dense compress / decompress, or the sparse
+operators with the straight-through gate scaling of `sparse_train`; dge.py:66-72, :91-106) are kept
+for API completeness: the router and the dense forms are plain differentiable torch ops there, the
+sparse operators use the kernels forward and backward.
 """
 import math
 from typing import List
 
 import torch
+import torch.nn.functional as F
 from torch import nn
 
 from .. import ops
-from .grained_sample import grained_sample_compress, grained_sample_decompress, grained_sample_index_to_patch
+from .grained_sample import (grained_sample_compress, grained_sample_compress_dense, grained_sample_decompress,
+                             grained_sample_decompress_dense, grained_sample_index_to_patch)
 
 
 class DynamicRouter(nn.Module):
@@ -50,6 +55,9 @@ class DynamicRouter(nn.Module):
     def forward(self, x):
         """x [B,H,W,C] -> gate logits [B,Hr,Wr,S] (the reference's call form, dge.py:145-150)."""
         B, H, W, C = x.shape
+        if self.training or torch.is_grad_enabled() and x.requires_grad:     # differentiable composition
+            pooled = F.avg_pool2d(x.permute(0, 3, 1, 2), self.region_size, self.region_size).permute(0, 2, 3, 1)
+            return self.gate(pooled)
         return self.route(x.reshape(B, H * W, C), H, W)[0]
 
 
@@ -86,11 +94,20 @@ class DynamicGrainedEncoder(nn.Module):
 
     def compress(self, x, H, W, gate=None):
         """x [B, extra+H*W, C] -> packed queries [L, C].  `gate` overrides the router output (tests)."""
-        if self.training:
-            raise NotImplementedError("only the inference branch of the Dynamic Grained Encoder is built")
         B, N, C = x.shape
         extra = N - H * W
-        if gate is None:
+        if self.training:
+            # dge.py:64-72: hard Gumbel sample of the gate; every granularity (dense) or the sampled one (sparse)
+            if gate is None:
+                gate = self.router(x[:, extra:, :].reshape(B, H, W, C))
+            gate = F.gumbel_softmax(gate, dim=-1, hard=True)
+            if not self.sparse_train:
+                comp, batches = grained_sample_compress_dense(x, self.splits, self.region_size, H, W, extra)
+                self.states.update({"comp": comp, "input": x, "patches": None, "batches": batches, "gate": gate,
+                                    "size": (H, W), "num_extra_tokens": extra})
+                return comp
+            indices = gate.argmax(dim=-1)
+        elif gate is None:
             gate, indices = self.router.route(x, H, W)
         else:
             indices = gate.argmax(dim=-1)
@@ -102,8 +119,18 @@ class DynamicGrainedEncoder(nn.Module):
 
     def decompress(self, x):
         """packed [L, C] -> tokens [B, N, C]: input + broadcast(x - comp).  dge.py:87-111."""
-        if self.training:
-            raise NotImplementedError("only the inference branch of the Dynamic Grained Encoder is built")
         st = self.states
-        return grained_sample_decompress(x - st["comp"], st["patches"], st["input"], *st["size"],
-                                         st["num_extra_tokens"], True)
+        x = x - st["comp"]
+        if self.training and not self.sparse_train:
+            return grained_sample_decompress_dense(x, st["gate"], st["input"], self.splits, self.region_size,
+                                                   *st["size"], st["num_extra_tokens"], True)
+        if self.training:
+            # dge.py:96-106: scale each query by its region's (hard, value 1) gate so the router receives a gradient
+            B, N, C = st["input"].shape
+            extra = st["num_extra_tokens"]
+            g = st["gate"].max(dim=-1, keepdim=True)[0]
+            g = g.repeat_interleave(self.region_size, 1).repeat_interleave(self.region_size, 2).reshape(B, -1, 1)
+            if extra > 0:
+                g = torch.cat([g.new_ones([B, extra, 1]), g], dim=1)
+            x = x * grained_sample_compress(g, st["patches"], *st["size"], extra)
+        return grained_sample_decompress(x, st["patches"], st["input"], *st["size"], st["num_extra_tokens"], True)

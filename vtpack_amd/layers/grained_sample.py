@@ -6,6 +6,7 @@ are the reference's (compress and decompress are adjoint up to size**2) expresse
 two kernels.
 """
 import torch
+import torch.nn.functional as F
 from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
@@ -85,3 +86,41 @@ grained_sample_compress = _Compress.apply
 grained_sample_decompress = _Decompress.apply
 grained_sample_index_to_patch = _IndexToPatch.apply
 grained_sample_index_to_patch_dense = _IndexToPatchDense.apply
+
+
+# ------------------------------------------------------------------ dense (training) forms
+def grained_sample_compress_dense(x, split_sizes, region_size, H, W, num_extra_tokens):
+    """Queries of EVERY granularity: the extra tokens, then for each split the whole grid pooled with that split's
+    window.  Plain torch ops (differentiable), as in the reference (vtpack/layers/grained_sample.py:126-148).
+    -> (comp [B * per_sample, C], batch_lengths int64 [B] on the CPU)."""
+    B, N, C = x.shape
+    grid = x[:, num_extra_tokens:, :].reshape(B, H, W, C).permute(0, 3, 1, 2)
+    levels = [x[:, :num_extra_tokens, :]] if num_extra_tokens > 0 else []
+    for ps in split_sizes.tolist():
+        step = region_size // int(ps)
+        pooled = F.avg_pool2d(grid, step, step) if step > 1 else grid
+        levels.append(pooled.flatten(2).transpose(1, 2))
+    comp = torch.cat(levels, dim=1)
+    return comp.reshape(-1, C), torch.full((B,), comp.shape[1], dtype=torch.int64)
+
+
+def grained_sample_decompress_dense(x, gate, reference, split_sizes, region_size, H, W, num_extra_tokens, is_add_ref):
+    """Inverse of the dense form: every level is upsampled to the token grid and the levels are mixed with the
+    per-region gate [B, Hr, Wr, S] (one-hot in the forward pass of training).
+    vtpack/layers/grained_sample.py:151-177."""
+    B, N, C = reference.shape
+    x = x.reshape(B, -1, C)
+    spatial = 0
+    start = num_extra_tokens
+    for i, ps in enumerate(split_sizes.tolist()):
+        step = region_size // int(ps)
+        Hi, Wi = H // step, W // step
+        level = x[:, start:start + Hi * Wi, :].reshape(B, Hi, Wi, C)
+        level = level.repeat_interleave(step, dim=1).repeat_interleave(step, dim=2)
+        weight = gate[..., i].repeat_interleave(region_size, dim=1).repeat_interleave(region_size, dim=2)
+        spatial = spatial + level * weight.unsqueeze(-1)
+        start += Hi * Wi
+    out = spatial.reshape(B, H * W, C)
+    if num_extra_tokens > 0:
+        out = torch.cat([x[:, :num_extra_tokens, :], out], dim=1)
+    return out + reference if is_add_ref else out
