@@ -4,6 +4,9 @@ Self-contained (no timm): the patch embedding is the Conv2d(3, C, 16, stride 16)
 wraps, DropPath/Dropout are identities at inference.  Sub-module and parameter names are the
 reference's, so its state dicts load with `load_state_dict` unchanged.
 
+In training mode a block runs the reference's training composition (Gumbel-sampled gate, dense or sparse
+operators, differentiable attention; deit_dge.py:79-95) with torch autograd around the operators.
+
 Every block can run two ways at inference:
   * layer mode  - the reference's composition (deit_dge.py:123-130): nn.LayerNorm / nn.Linear from
     torch around the `vtpack.layers` operators, one device->host copy of the query counts per block;
@@ -18,7 +21,7 @@ from torch import nn
 
 from ... import engine
 from ...layers import DynamicGrainedEncoder
-from ...layers.sparse_ops import batched_sparse_attention
+from ...layers.sparse_ops import batched_sparse_attention, sparse_attention_train
 
 __all__ = ["VisionTransformer", "Block", "Attention", "Mlp", "PatchEmbed", "deit_dge_s124_tiny_patch16_256",
            "deit_dge_s124_small_patch16_256", "deit_dge_s124_base_patch16_256"]
@@ -58,13 +61,13 @@ class Attention(nn.Module):
                 + 3 * num_queries * num_inputs * self.num_heads + num_queries * c * c)
 
     def forward(self, x, q, q_lengths):
-        # deit_dge.py:70-78,96 (inference branch)
-        if self.training:
-            raise NotImplementedError("only the inference branch is built")
+        # deit_dge.py:70-78,96 
         B, N, C = x.shape
         h, d = self.num_heads, C // self.num_heads
         q = self.q(q).reshape(-1, h, d).permute(1, 0, 2)
         kv = self.kv(x).reshape(B, N, 2, h, d).permute(2, 3, 0, 1, 4)
+        if self.training:
+            return self.proj(sparse_attention_train(q, kv[0], kv[1], q_lengths, self.scale))
         o = batched_sparse_attention(q, kv[0], kv[1], q_lengths, self.scale)
         return self.proj(o.transpose(0, 1).reshape(-1, C))
 
