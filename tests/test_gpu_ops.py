@@ -9,7 +9,7 @@ import torch
 
 from oracle import dge_oracle as orc
 from oracle import torch_ref
-from util import SPLITS, assert_close, bf16_round, randn, random_indices, rel_err, rng
+from util import BF16_ABS, SPLITS, abs_err, assert_close, bf16_round, randn, random_indices, rel_err, rng
 
 pytestmark = pytest.mark.gpu
 
@@ -207,6 +207,71 @@ def test_linear_device_rows(dev):
     want = torch.from_numpy(a[:live]).double() @ torch.from_numpy(w).double().T
     assert rel_err(out[:live], want) <= 1e-5
     assert bool((out[live:] == 7.0).all())
+
+
+# The packed Linear of the C = 384 models in bf16 (K = 384, N a multiple of 384, >= 2048 rows) runs on the
+# weight-stationary kernel: ragged last tiles, fewer tiles than workgroups, several column groups, every epilogue,
+# live row count on the device.
+@pytest.mark.parametrize("M,N", [(2048, 384), (2049, 768), (4127, 384), (9000, 1152), (33000, 1536), (70000, 768)])
+@pytest.mark.parametrize("epi", ["plain", "bias", "bias_gelu", "bias_res", "gelu_res", "bias_gelu_res"])
+def test_linear_weight_stationary(dev, M, N, epi):
+    from vtpack_amd import ops
+    if M > 40000 and epi not in ("bias", "bias_res"):
+        pytest.skip("largest shape: the two epilogues of the model are enough")
+    K = 384
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16()
+    res = torch.randn(M, N, generator=g).bfloat16()
+    want = a.double() @ w.double().T
+    if "bias" in epi:
+        want = want + bias.double()
+    if "gelu" in epi:
+        want = torch.nn.functional.gelu(want)
+    if "res" in epi:
+        want = want + res.double()
+    got = ops.linear(a.to(dev), w.to(dev), bias.to(dev) if "bias" in epi else None,
+                     res.to(dev) if "res" in epi else None, act="gelu" if "gelu" in epi else "none")
+    # one bf16 rounding of a value of magnitude up to ~8: half an ulp is 2^-6; the bar of the other bf16 tests
+    # (2e-2) is kept on everything below 4
+    err = (got.double().cpu() - want).abs()
+    small = want.abs() < 4
+    assert float(err[small].max()) <= BF16_ABS, f"weight-stationary linear {epi}: {float(err[small].max()):.3e}"
+    assert float((err / want.abs().clamp_min(4)).max()) <= 2 ** -7, f"weight-stationary linear {epi} (relative)"
+
+
+def test_linear_weight_stationary_device_rows(dev):
+    from vtpack_amd import ops
+    M, N, K, live = 6000, 768, 384, 4999
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    res = torch.randn(M, N, generator=g).bfloat16()
+    rows_dev = torch.tensor([live], dtype=torch.int64, device=dev)
+    out = torch.full((M, N), 7.0, device=dev, dtype=torch.bfloat16)
+    ops.linear(a.to(dev), w.to(dev), residual=res.to(dev), rows_dev=rows_dev, out=out)
+    want = a[:live].double() @ w.double().T + res[:live].double()
+    assert abs_err(out[:live], want) <= 4 * BF16_ABS        # values up to ~10: one bf16 rounding
+    assert bool((out[live:] == 7.0).all())
+    # a live count of zero touches nothing
+    out.fill_(7.0)
+    ops.linear(a.to(dev), w.to(dev), rows_dev=torch.zeros(1, dtype=torch.int64, device=dev), out=out)
+    assert bool((out == 7.0).all())
+
+
+def test_linear_weight_stationary_matches_streaming_kernel(dev):
+    """Both bf16 kernels accumulate the K dimension in the same order in fp32, so they agree bit for bit; fewer
+    than 2048 rows send the same rows to the streaming kernel."""
+    from vtpack_amd import ops
+    M, N, K = 5003, 768, 384
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev)
+    got = ops.linear(a, w, bias, act="gelu")
+    few = ops.linear(a[:2000], w, bias, act="gelu")          # < 2048 rows: streaming kernel
+    assert torch.equal(got[:2000], few)
 
 
 # ------------------------------------------------------------------ attention / sparse gemm

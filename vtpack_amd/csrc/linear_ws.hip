@@ -1,0 +1,527 @@
+// Packed-M Linear for bf16 operands with a short K (K * 2 bytes = 768: the C = 384 models), weight-stationary.
+//
+// A workgroup is 4 waves, one per SIMD, and owns a strip of BN = 4 * NB * 32 output columns for its whole life:
+// every wave keeps its NB * 32 rows of W (all of K) in registers as ready-made MFMA operands (NB * K/16 fragments
+// of 4 registers: 288 for NB = 3, K = 384; half of them in accumulation registers, which the MFMA reads directly),
+// so the only operand that moves while the kernel runs is A.
+// A streams HBM/L2 -> LDS in 32-row tiles by direct loads (no VGPR staging) into a ring that is several tiles
+// deep; each wave multiplies every A tile against its own columns:  D = W_strip * A_tile^T, 32 x 32 x 16 MFMAs,
+// so a lane owns one output row and bias / GELU / residual are applied in fp32 on 8-column vectors.
+// Per output tile the memory system delivers 24 KB for 72 MFMAs per wave: ~10 B/clk per CU, against the ~46
+// B/clk a CU can pull from L2, and the MFMA pipe never waits on the second operand.
+//
+// With one wave per SIMD nothing overlaps by itself, so the instruction stream is woven by hand: the fragment of
+// A for substep s+3 is read from LDS before the MFMAs of substep s, and the epilogue of tile t (24 units of two
+// output elements per lane) is spread over the 24 substeps of tile t+1, which accumulates into a second register
+// set; a few vector instructions follow each MFMA and run while it executes.
+//
+// W reaches the registers through LDS as well (before the first A tile needs the space): coalesced direct loads of
+// 32-row blocks in the same slab layout as A, two half-rings of three blocks, each wave reading its own blocks as
+// fragments while the next blocks are in flight.
+//
+// Synchronisation: one s_barrier per tile.  Vector-memory operations retire in issue order, so before the barrier
+// a wave waits with a *counted* s_waitcnt vmcnt until its own direct loads of the tile about to be consumed have
+// landed; younger prefetches and stores stay in flight.  The count is kept exactly: a per-wave tally of issued
+// operations and, per tile, the tally right after its loads.  The direct loads and the MFMAs are issued from inline
+// assembly (the LDS reads of the fragments then need no vmcnt wait of the compiler's own, and the stationary
+// fragments stay where they were put).
+//
+// Rows >= M of the last tile are clamped to row M-1 on every read and on the store: those lanes recompute row M-1
+// bit for bit and store the same bytes, so the tile loop has no predicated memory operation.
+#include "common.h"
+#include <stdlib.h>
+#include <type_traits>
+
+namespace vtdge {
+
+#ifdef VT_WS_DEBUG
+__device__ long long ws_dbg[4][64];
+#define VT_WS_STAMP(i)                                                                         \
+    do {                                                                                       \
+        if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100) && (i) < 64)                     \
+            ws_dbg[blockIdx.x == 0 ? 0 : 1][(i)] = clock64();                                  \
+    } while (0)
+#else
+#define VT_WS_STAMP(i) do { } while (0)
+#endif
+
+// one direct load: 64 lanes x 16 B from base + the per-lane byte offset to LDS bytes [lds_addr, lds_addr + 1024)
+__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base)
+                 : "memory", "m0");
+}
+// makes a lane constant opaque at this point, so address arithmetic built on it is redone where it is used instead
+// of being kept in registers for the whole kernel
+__device__ __forceinline__ int fresh(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+// D = W_frag * A_frag^T (+ D).  The stationary fragment sits in accumulation registers (A) or vector registers (V);
+// Z starts a new sum.  Issued from assembly so the register classes are exactly these.
+__device__ __forceinline__ void mma_a(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(d) : "a"(wfrag), "v"(afrag));
+}
+__device__ __forceinline__ void mma_v(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(d) : "v"(wfrag), "v"(afrag));
+}
+__device__ __forceinline__ void mma_az(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
+{
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(d) : "a"(wfrag), "v"(afrag));
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform runtime n (a multiple of 6; more than 60 waits for 60)
+__device__ __forceinline__ void wait_vmcnt_dyn(int n)
+{
+    switch (n / 6) {
+    case 0: wait_vmcnt<0>(); break;
+    case 1: wait_vmcnt<6>(); break;
+    case 2: wait_vmcnt<12>(); break;
+    case 3: wait_vmcnt<18>(); break;
+    case 4: wait_vmcnt<24>(); break;
+    case 5: wait_vmcnt<30>(); break;
+    case 6: wait_vmcnt<36>(); break;
+    case 7: wait_vmcnt<42>(); break;
+    case 8: wait_vmcnt<48>(); break;
+    case 9: wait_vmcnt<54>(); break;
+    default: wait_vmcnt<60>(); break;
+    }
+}
+
+// State of one epilogue unit: two output elements of a lane on their way from the accumulator to bf16.
+struct EpiUnit {
+    float f0, f1;   // values
+    float x0, x1, t0, t1, q0, q1;   // GELU: clamped argument, its square, Horner accumulator
+};
+
+// GELU(x) = x * Phi(x), Phi - 1/2 as a degree-15 odd minimax polynomial on [-4, 4] (x clamped there):
+// |error| <= 1.3e-4, below 1/30 of a bf16 rounding step of the result.  Three parts of about equal length.
+__device__ __forceinline__ void gelu_part1(EpiUnit &u)
+{
+    u.x0 = __builtin_amdgcn_fmed3f(u.f0, -4.0f, 4.0f);
+    u.x1 = __builtin_amdgcn_fmed3f(u.f1, -4.0f, 4.0f);
+    u.t0 = u.x0 * u.x0;
+    u.t1 = u.x1 * u.x1;
+    u.q0 = -1.580785487e-09f * u.t0 + 1.217110604e-07f;
+    u.q1 = -1.580785487e-09f * u.t1 + 1.217110604e-07f;
+    u.q0 = u.q0 * u.t0 - 4.100865225e-06f;
+    u.q1 = u.q1 * u.t1 - 4.100865225e-06f;
+}
+__device__ __forceinline__ void gelu_part2(EpiUnit &u)
+{
+    u.q0 = u.q0 * u.t0 + 8.066737963e-05f;
+    u.q1 = u.q1 * u.t1 + 8.066737963e-05f;
+    u.q0 = u.q0 * u.t0 - 1.048204291e-03f;
+    u.q1 = u.q1 * u.t1 - 1.048204291e-03f;
+    u.q0 = u.q0 * u.t0 + 9.664873803e-03f;
+    u.q1 = u.q1 * u.t1 + 9.664873803e-03f;
+    u.q0 = u.q0 * u.t0 - 6.617537860e-02f;
+    u.q1 = u.q1 * u.t1 - 6.617537860e-02f;
+}
+__device__ __forceinline__ void gelu_part3(EpiUnit &u)
+{
+    u.q0 = u.q0 * u.t0 + 3.988475095e-01f;
+    u.q1 = u.q1 * u.t1 + 3.988475095e-01f;
+    u.f0 = u.f0 * (u.x0 * u.q0 + 0.5f);
+    u.f1 = u.f1 * (u.x1 * u.q1 + 0.5f);
+}
+
+template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES>
+__global__ __launch_bounds__(256) void linear_ws_kernel(
+    const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
+    const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
+    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P)
+{
+    constexpr int KB = KS * 32;                 // bytes of one operand row
+    constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
+    constexpr int STRIP = NB * 32;              // output columns per wave
+    constexpr int BN = 4 * STRIP;               // output columns per workgroup
+    constexpr int RROW = BN * 2;                // bytes of one residual row of the strip
+    constexpr int DA = HAS_RES ? 3 : 6;         // A ring depth (tiles)
+    constexpr int DR = 3;                       // residual ring depth
+    constexpr int PA = DA - 1;                  // A tiles in flight ahead of the one being multiplied
+    constexpr int NL = TILE / 1024 / 4;         // direct loads per wave and tile
+    constexpr int NU = NB * 8;                  // epilogue units per tile (two elements each)
+    constexpr int KA = KS / 2 + 1;                 // substeps whose W fragments live in accumulation registers
+    static_assert(KS % 4 == 0 && NL * 4 * 1024 == TILE && 32 * RROW == TILE, "tile geometry");
+    static_assert(NL == 6 && NB == 3, "the vmcnt bookkeeping counts in units of 6");
+    static_assert(NU == KS, "one epilogue unit per K substep");
+    static_assert(RROW % 256 == 0 && STRIP % 16 == 0, "residual tile: column groups of 256 B");
+    constexpr int EARLY = HAS_RES ? 1 : 3;      // A tiles issued while the last W blocks are still being read
+    constexpr int OFF_R = DA * TILE;
+    constexpr int OFF_B = 6 * TILE;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+
+    const int64_t M = live_rows(rows_dev, rows);
+    const int tiles_m = (int)((M + 31) / 32);
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int g = slot % groups;                     // column group
+    const int p = xcd + 8 * (slot / groups);         // position among the P workgroups of the group
+    const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
+    if (nt == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    VT_WS_STAMP(0);
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 31, lg = lane >> 5;
+    const int col0 = g * BN + w * STRIP;             // first output column of this wave
+
+    // ---- per-lane constants
+    // fragment reads: row lr of the tile, 16-byte chunk (2c + lg) of a 128-byte slab, slot-swizzled
+    int cs[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) cs[c] = lr * 128 + (((2 * c + lg) ^ ((lr >> 1) & 7)) * 16);
+    // direct loads of a 32-row operand tile (A or a W block): instruction i = w*NL + ii covers slab i/4 and rows
+    // (i%4)*8 + lane/8; the lane fetches chunk (lane%8) ^ ((row/2)%8) = ((lane%8) ^ (lane/16)) ^ 4*(i%2).
+    // Everything that depends on i is wave-uniform, so two lane constants serve all of a wave's loads.
+    const int l8 = lane >> 3;
+    const int ax16 = ((lane & 7) ^ (lane >> 4)) * 16;
+    auto a_row = [&](int ii, int l8v) -> int { return ((w * NL + ii) & 3) * 8 + l8v; };
+    auto a_off = [&](int ii, int ax16v) -> int { const int i = w * NL + ii; return (i >> 2) * 128 + (ax16v ^ ((i & 1) * 64)); };
+    // the residual tile: 32 rows x RROW bytes as RROW/256 column groups of [32 rows][256 B]; instruction i covers
+    // group i/8 and rows (i%8)*4 + lane/16; inside a row the sixteen 16-byte chunks are XOR-swizzled with the row,
+    // so the epilogue's reads (16 rows at one column) are conflict free.
+    const int l16 = lane >> 4;
+    const int ry16 = ((lane & 15) ^ (lane >> 4)) * 16;
+    auto r_row = [&](int ii, int l16v) -> int { return ((w * NL + ii) & 7) * 4 + l16v; };
+    auto r_off = [&](int ii, int ry16v) -> int { const int i = w * NL + ii; return g * RROW + (i >> 3) * 256 + (ry16v ^ ((i & 3) * 64)); };
+    // epilogue: lane (lr, lg) handles row lr and the 8-column vector (j, q) = chunk cb + lg, cb = 12*w + 4*j + 2*q
+    const int ebase = lr * 256 + ((lg ^ (lr & 15)) * 16);
+    auto e_roff = [&](int j, int q) -> int { const int cb = w * (STRIP / 8) + j * 4 + q * 2; return (cb >> 4) * 8192 + (ebase ^ ((cb & 15) * 16)); };
+    const int lg16 = lg * 16;
+
+    const int M32 = (int)M;
+    const uint32_t lda2 = (uint32_t)lda * 2, ldr2 = (uint32_t)ldr * 2, ldo2 = (uint32_t)ldo * 2;   // row pitches, bytes
+    auto tile_row0 = [&](int k) -> int { return (p + k * P) * 32; };
+
+    // tally of vector-memory operations issued by this wave and, per A tile, the tally right after its loads
+    int issued = 0;
+    uint64_t marks = 0;
+    auto issue_a = [&](int k) {
+        const int m0 = tile_row0(k);
+        const uint32_t dst = lds0 + (k % DA) * TILE + w * NL * 1024;
+        const int l8v = fresh(l8), ax16v = fresh(ax16);
+#pragma unroll
+        for (int ii = 0; ii < NL; ii++) {
+            int gm = m0 + a_row(ii, l8v);
+            gm = gm < M32 ? gm : M32 - 1;
+            dma16(A, (uint32_t)gm * lda2 + a_off(ii, ax16v), dst + ii * 1024);
+        }
+        issued += NL;
+        const int sh = (k & 7) * 8;
+        marks = (marks & ~(0xffull << sh)) | ((uint64_t)(issued & 0xff) << sh);
+    };
+    auto issue_r = [&](int k) {
+        const int m0 = tile_row0(k);
+        const uint32_t dst = lds0 + OFF_R + (k % DR) * TILE + w * NL * 1024;
+        const int l16v = fresh(l16), ry16v = fresh(ry16);
+#pragma unroll
+        for (int ii = 0; ii < NL; ii++) {
+            int gm = m0 + r_row(ii, l16v);
+            gm = gm < M32 ? gm : M32 - 1;
+            dma16(res, (uint32_t)gm * ldr2 + r_off(ii, ry16v), dst + ii * 1024);
+        }
+        issued += NL;
+    };
+
+    // ---- the stationary operand: 12 blocks of 32 W rows (block = 3 * wave + j) pass through the six LDS slots,
+    // three at a time; wave `r` picks its fragments out of round r.
+    u32x4 wfa[NB][KA], wfv[NB][KS - KA];
+    {
+        auto issue_w = [&](int round) {   // blocks 3*round .. 3*round+2 -> slots 3*(round&1) ..
+#pragma unroll
+            for (int b = 0; b < 3; b++) {
+                const uint32_t src = (uint32_t)(g * BN + (round * 3 + b) * 32) * KB;
+                const uint32_t dst = lds0 + ((round & 1) * 3 + b) * TILE + w * NL * 1024;
+#pragma unroll
+                for (int ii = 0; ii < NL; ii++) dma16(Wt, src + a_row(ii, l8) * KB + a_off(ii, ax16), dst + ii * 1024);
+            }
+        };
+        auto read_w = [&](int round) {
+            const unsigned char *base = smem + (round & 1) * 3 * TILE;
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+#pragma unroll
+                for (int s = 0; s < KS; s++) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(base + j * TILE + (s >> 2) * 4096 + cs[s & 3]);
+                    if (s < KA) wfa[j][s] = v;
+                    else wfv[j][s - KA] = v;
+                }
+        };
+        if constexpr (HAS_BIAS) {
+            // the strip's bias: one direct load by wave 0, the oldest operation of all (lanes past the strip re-read
+            // its last chunk; the LDS area is a full 1 KB)
+            if (w == 0) {
+                const int c = lane < BN / 8 ? lane : BN / 8 - 1;
+                dma16(bias, (uint32_t)(g * BN * 2 + c * 16), lds0 + OFF_B);
+            }
+        }
+        issue_w(0);
+        issue_w(1);
+#pragma unroll
+        for (int round = 0; round < 4; round++) {
+            if (round < 3) wait_vmcnt<3 * NL>();   // everything but the youngest round has landed
+            else wait_vmcnt_dyn(issued);           // ... but the first A tiles
+            __syncthreads();
+            if (w == round) read_w(round);
+            __syncthreads();                       // the three slots are free again
+            if (round + 2 < 4) issue_w(round + 2);
+            if (round == 2) {
+                // slots 0..2 have seen their last W block: the first A tiles can follow
+#pragma unroll
+                for (int k = 0; k < EARLY; k++)
+                    if (k < nt) issue_a(k);
+            }
+        }
+    }
+    VT_WS_STAMP(1);
+
+    f32x16 acc[2][NB];
+
+    // ---- epilogue of one tile, in NU units.  Unit n = 4 * (2j + q) + e turns the accumulator pair
+    // (8q + e, 8q + 4 + e) of block j into elements e and 4 + e of the lane's 8-column vector (j, q).
+    // Bias and residual of a vector come from LDS.  The residual (used last in a unit) is fetched right after the
+    // previous vector is stored; so is the bias when it is added last too (no activation) or when registers are
+    // short (activation + residual); otherwise the bias is fetched one unit ahead into a second register set.
+    constexpr bool LATE_BIAS = ACT == VTDGE_ACT_NONE || HAS_RES;
+    constexpr bool BIAS_LAST = ACT == VTDGE_ACT_NONE;
+    u32x4 e_bias, e_res, n_bias;
+    uint32_t e_w[4];        // packed pairs of the current vector
+    float h0, h1;           // elements of an even unit waiting for their odd neighbours
+    EpiUnit un;
+    auto fetch_bias = [&](u32x4 &dst, int vec) {
+        dst = *reinterpret_cast<const u32x4 *>(smem + OFF_B + (w * (STRIP / 8) + (vec / 2) * 4 + (vec % 2) * 2) * 16 + lg16);
+    };
+    auto fetch_res = [&](int k, int vec) {
+        e_res = *reinterpret_cast<const u32x4 *>(smem + OFF_R + (k % DR) * TILE + e_roff(vec / 2, vec % 2));
+    };
+    auto epi_begin = [&](int k) {     // LDS reads for vector 0 of tile k
+        if constexpr (HAS_BIAS) fetch_bias(LATE_BIAS ? e_bias : n_bias, 0);
+        if constexpr (HAS_RES) fetch_res(k, 0);
+    };
+    auto word_lo_hi = [](const u32x4 &v, int e) -> float {   // element e (0..7) of a vector of 8 bf16
+        const uint32_t wd = v[e / 2];
+        return (e & 1) ? bf16hi(wd) : bf16lo(wd);
+    };
+    // part 1 of unit n: out of the accumulator, bias, first third of the activation
+    auto epi_part1 = [&](auto pp_tag, int n) {
+        constexpr int PP = decltype(pp_tag)::value;
+        const int j = n / 8, q = (n / 4) % 2, e = n % 4;
+        if constexpr (HAS_BIAS && !LATE_BIAS) {
+            if (e == 0) e_bias = n_bias;
+        }
+        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[PP][j][8 * q + e]),
+                                                  __float_as_uint(acc[PP][j][8 * q + 4 + e]), false, false);
+        un.f0 = __uint_as_float(r[0]);
+        un.f1 = __uint_as_float(r[1]);
+        if constexpr (HAS_BIAS && !BIAS_LAST) {
+            un.f0 += word_lo_hi(e_bias, e);
+            un.f1 += word_lo_hi(e_bias, 4 + e);
+        }
+        if constexpr (ACT == VTDGE_ACT_GELU) gelu_part1(un);
+    };
+    auto epi_part2 = [&](int n) {
+        if constexpr (ACT == VTDGE_ACT_GELU) gelu_part2(un);
+    };
+    // part 3: rest of the activation, residual; odd units pack, the fourth unit of a vector stores it
+    auto epi_part3 = [&](int k, int n, unsigned char *orow) {
+        const int j = n / 8, q = (n / 4) % 2, e = n % 4;
+        if constexpr (ACT == VTDGE_ACT_GELU) gelu_part3(un);
+        if constexpr (HAS_BIAS && BIAS_LAST) {
+            un.f0 += word_lo_hi(e_bias, e);
+            un.f1 += word_lo_hi(e_bias, 4 + e);
+        }
+        if constexpr (HAS_RES) {
+            un.f0 += word_lo_hi(e_res, e);
+            un.f1 += word_lo_hi(e_res, 4 + e);
+        }
+        if (e % 2 == 0) {
+            h0 = un.f0;
+            h1 = un.f1;
+        } else {
+            e_w[e / 2] = pack_bf16x2(h0, un.f0);        // elements e-1, e
+            e_w[2 + e / 2] = pack_bf16x2(h1, un.f1);    // elements 4+e-1, 4+e
+        }
+        if constexpr (HAS_BIAS && !LATE_BIAS) {
+            if (e == 2 && n + 2 < NU) fetch_bias(n_bias, n / 4 + 1);
+        }
+        if (e == 3) {
+            u32x4 v;
+            v.x = e_w[0]; v.y = e_w[1]; v.z = e_w[2]; v.w = e_w[3];
+            *reinterpret_cast<u32x4 *>(orow + (j * 32 + 8 * 2 * q) * 2) = v;
+            if (n + 1 < NU) {
+                if constexpr (HAS_BIAS && LATE_BIAS) fetch_bias(e_bias, n / 4 + 1);
+                if constexpr (HAS_RES) fetch_res(k, n / 4 + 1);
+            }
+        }
+    };
+    auto out_row = [&](int k) -> unsigned char * {
+        int gm = tile_row0(k) + lr;
+        gm = gm < M32 ? gm : M32 - 1;
+        return reinterpret_cast<unsigned char *>(out) + (uint64_t)(uint32_t)gm * ldo2 + (col0 + 8 * lg) * 2;
+    };
+
+    // ---- one tile: wait for A(k), multiply into acc[PP]; when EPI, finish tile k-1 (in acc[1-PP]) on the way
+    auto tile_step = [&](auto pp_tag, auto epi_tag, int k) {
+        constexpr int PP = decltype(pp_tag)::value;
+        constexpr bool EPI = decltype(epi_tag)::value;
+        using PQ = std::integral_constant<int, 1 - PP>;
+        const int after = (issued - (int)((marks >> ((k & 7) * 8)) & 0xff)) & 0xff;
+        VT_WS_STAMP(3 + 2 * k);
+        wait_vmcnt_dyn(after);
+        VT_WS_STAMP(4 + 2 * k);
+        block_barrier();   // A(k) (and the residual of k-1) are in LDS for every wave; the slots read last step are free
+        if constexpr (HAS_RES) {
+            if (k + 1 < nt) issue_r(k + 1);
+        }
+        if (k + PA < nt) issue_a(k + PA);
+
+        const unsigned char *at = smem + (k % DA) * TILE;
+        unsigned char *orow = nullptr;
+        if constexpr (EPI) {
+            orow = out_row(k - 1);
+            epi_begin(k - 1);
+        }
+        // fragments of A are read FD substeps ahead of the MFMAs that use them
+        constexpr int FD = HAS_RES ? 2 : 3;
+        u32x4 fa[FD + 1];
+#pragma unroll
+        for (int s = 0; s < FD; s++) fa[s] = *reinterpret_cast<const u32x4 *>(at + (s >> 2) * 4096 + cs[s & 3]);
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            if (s + FD < KS)
+                fa[(s + FD) % (FD + 1)] =
+                    *reinterpret_cast<const u32x4 *>(at + ((s + FD) >> 2) * 4096 + cs[(s + FD) & 3]);
+            __builtin_amdgcn_sched_barrier(0);   // keep the read ahead of, not next to, its use
+            const u32x4 &f = fa[s % (FD + 1)];
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                if (s == 0) mma_az(acc[PP][j], wfa[j][0], f);
+                else if (s < KA) mma_a(acc[PP][j], wfa[j][s], f);
+                else mma_v(acc[PP][j], wfv[j][s - KA], f);
+                if constexpr (EPI) {
+                    // a few vector instructions behind every MFMA: they execute while it runs
+                    if (j == 0) epi_part1(PQ{}, s);
+                    if (j == 1) epi_part2(s);
+                    if (j == 2) epi_part3(k - 1, s, orow);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        if constexpr (EPI) issued += NB * 2;
+    };
+
+    // ---- rest of the prologue: first residual tile (ahead of A(1): a tile's wait covers what was issued before it),
+    // remaining first tiles of A
+    if constexpr (HAS_RES) issue_r(0);
+#pragma unroll
+    for (int k = EARLY; k < PA; k++)
+        if (k < nt) issue_a(k);
+
+    VT_WS_STAMP(2);
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    tile_step(I0{}, std::false_type{}, 0);
+    int k = 1;
+    for (; k + 1 < nt; k += 2) {
+        tile_step(I1{}, std::true_type{}, k);
+        tile_step(I0{}, std::true_type{}, k + 1);
+    }
+    if (k < nt) {
+        tile_step(I1{}, std::true_type{}, k);
+        k++;
+    }
+    VT_WS_STAMP(3 + 2 * nt);
+    // ---- last tile's epilogue (its residual was fetched two steps ago: wait for everything, publish)
+    wait_vmcnt<0>();
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs' results must have reached the registers
+    block_barrier();
+    unsigned char *orow = out_row(nt - 1);
+    epi_begin(nt - 1);
+    if ((nt - 1) & 1) {
+#pragma unroll
+        for (int n = 0; n < NU; n++) {
+            epi_part1(I1{}, n);
+            epi_part2(n);
+            epi_part3(nt - 1, n, orow);
+        }
+    } else {
+#pragma unroll
+        for (int n = 0; n < NU; n++) {
+            epi_part1(I0{}, n);
+            epi_part2(n);
+            epi_part3(nt - 1, n, orow);
+        }
+    }
+    VT_WS_STAMP(4 + 2 * nt);
+}
+
+// ----------------------------------------------------------------------------- host
+bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, const void *bias,
+                          const void *res, const void *out)
+{
+    static int off = -1;   // VTDGE_LINEAR_WS=0 keeps these shapes on the streaming kernel (A/B timing)
+    if (off < 0) {
+        const char *e = getenv("VTDGE_LINEAR_WS");
+        off = (e && atoi(e) == 0) ? 1 : 0;
+    }
+    if (off) return false;
+    return esz == 2 && K == 384 && lda < (1ll << 31) && ldo < (1ll << 31) && ldr < (1ll << 31) && N % 384 == 0 &&
+           N / 384 <= 8 && rows >= 2048 && rows * lda < (1ll << 31) && (res == nullptr || rows * ldr < (1ll << 31)) && lda % 8 == 0 && ldo % 8 == 0 &&
+           (res == nullptr || ldr % 8 == 0) && (((uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15) == 0;
+}
+
+template <int ACT, bool HB, bool HR>
+static int go_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr, void *out,
+                 int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
+{
+    constexpr int KS = 24, NB = 3;
+    constexpr size_t lds = (size_t)6 * 32 * KS * 32 + 1024;   // six 32-row tiles + the strip's bias
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR>;
+    static bool attr_done = false;  // one flag per instantiation
+    if (!attr_done) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            set_error("linear: cannot reserve %zu bytes of LDS", lds);
+            return VTDGE_ERR_LAUNCH;
+        }
+        attr_done = true;
+    }
+    const int groups = N / (4 * NB * 32);
+    // one workgroup per CU; the P workgroups of a column group are spread over the 8 XCDs, and the workgroups
+    // that share A tiles (same position in different groups) sit on the same XCD
+    int P = (256 / groups) & ~7;
+    const int64_t tiles_m = ceil_div(rows, 32);
+    if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
+    dim3 grid((unsigned)(P * groups)), block(256);
+    kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
+                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P);
+    return check_launch("linear");
+}
+
+int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
+                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act, hipStream_t st)
+{
+    const bool hb = bias != nullptr, hr = res != nullptr;
+#define VT_WS(ACT, HB, HR) return go_ws<ACT, HB, HR>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st)
+    if (act == VTDGE_ACT_GELU) {
+        if (hb && hr) VT_WS(VTDGE_ACT_GELU, true, true);
+        if (hb) VT_WS(VTDGE_ACT_GELU, true, false);
+        if (hr) VT_WS(VTDGE_ACT_GELU, false, true);
+        VT_WS(VTDGE_ACT_GELU, false, false);
+    }
+    if (hb && hr) VT_WS(VTDGE_ACT_NONE, true, true);
+    if (hb) VT_WS(VTDGE_ACT_NONE, true, false);
+    if (hr) VT_WS(VTDGE_ACT_NONE, false, true);
+    VT_WS(VTDGE_ACT_NONE, false, false);
+#undef VT_WS
+}
+
+}  // namespace vtdge
