@@ -69,7 +69,9 @@ def kernel_symbol(name, tag, dt, n_keys=0):
     b = lambda v: "true" if v else "false"  # noqa: E731
     if name == "vtdge_linear":
         act = 1 if tag[1] == "gelu" else 0
-        N, K = tag[5], tag[6]
+        rows, N, K = tag[4], tag[5], tag[6]
+        if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
+            return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}>"

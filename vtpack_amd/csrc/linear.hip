@@ -194,8 +194,8 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
                       hipStream_t st);
 
 // weight-stationary variant for bf16, K = 384 (linear_ws.hip)
-bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, const void *bias,
-                          const void *res, const void *out);
+bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
+                          const void *bias, const void *res, const void *out);
 int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
                      void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act, hipStream_t st);
 
@@ -220,7 +220,7 @@ extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const voi
                "linear: A and W must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (linear_ws_applicable(lda, ldr, ldo, rows, N, K, esz, bias, residual, out))
+    if (linear_ws_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
         return launch_linear_ws(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
     if (linear_dma_applicable(lda, ldr, ldo, N, K, esz, bias, residual, out)) {
         if (dtype == VTDGE_F32)

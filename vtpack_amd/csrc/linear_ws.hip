@@ -63,15 +63,21 @@ __device__ __forceinline__ int fresh(int v)
 // Z starts a new sum.  Issued from assembly so the register classes are exactly these.
 __device__ __forceinline__ void mma_a(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
 {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(d) : "a"(wfrag), "v"(afrag));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "a"(wfrag), "v"(afrag));
 }
 __device__ __forceinline__ void mma_v(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
 {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(d) : "v"(wfrag), "v"(afrag));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(wfrag), "v"(afrag));
+}
+// for operands written by vector instructions just before: the two wait states the MFMA needs after such a write
+// (the compiler adds them for its own MFMAs, not inside assembly)
+__device__ __forceinline__ void mma_v_fresh(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
+{
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(wfrag), "v"(afrag));
 }
 __device__ __forceinline__ void mma_az(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
 {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(d) : "a"(wfrag), "v"(afrag));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "a"(wfrag), "v"(afrag));
 }
 
 // s_waitcnt vmcnt(n) for a wave-uniform runtime n (a multiple of 6; more than 60 waits for 60)
@@ -140,20 +146,25 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
     constexpr int STRIP = NB * 32;              // output columns per wave
     constexpr int BN = 4 * STRIP;               // output columns per workgroup
-    constexpr int RROW = BN * 2;                // bytes of one residual row of the strip
-    constexpr int DA = HAS_RES ? 3 : 6;         // A ring depth (tiles)
-    constexpr int DR = 3;                       // residual ring depth
-    constexpr int PA = DA - 1;                  // A tiles in flight ahead of the one being multiplied
+    constexpr int DA = HAS_RES ? 3 : 6;         // A ring depth (tiles); the residual ring takes the other three slots
+    constexpr int DR = 3;
+    constexpr int PA = DA - 1;                  // step k issues the loads of A(k + PA)
+    constexpr int PR = DR - 1;                  // ... and of the residual of tile k + PR
+    // Without a residual a step waits for the tile after its own, whose first fragments it reads at its end, so no
+    // MFMA waits for LDS behind the barrier; with only two tiles of A in flight that wait would come too early.
+    constexpr bool XT = !HAS_RES;
     constexpr int NL = TILE / 1024 / 4;         // direct loads per wave and tile
     constexpr int NU = NB * 8;                  // epilogue units per tile (two elements each)
-    constexpr int KA = KS / 2 + 1;                 // substeps whose W fragments live in accumulation registers
-    static_assert(KS % 4 == 0 && NL * 4 * 1024 == TILE && 32 * RROW == TILE, "tile geometry");
+    constexpr int KA = KS - 3;                  // substeps whose W fragments live in accumulation registers
+    constexpr int FD = (HAS_RES || ACT != VTDGE_ACT_NONE) ? 2 : 3;         // fragments of A are read FD substeps ahead of their MFMAs
+    constexpr int EARLY = PA < 3 ? PA : 3;      // A tiles issued while the last W blocks are still being read
+    static_assert(KS % 4 == 0 && NL * 4 * 1024 == TILE && BN * 2 == KB, "tile geometry (residual rows = A rows)");
+    static_assert(!(HAS_RES && ACT != VTDGE_ACT_NONE), "the residual is summed in the accumulator, ahead of an activation");
     static_assert(NL == 6 && NB == 3, "the vmcnt bookkeeping counts in units of 6");
     static_assert(NU == KS, "one epilogue unit per K substep");
-    static_assert(RROW % 256 == 0 && STRIP % 16 == 0, "residual tile: column groups of 256 B");
-    constexpr int EARLY = HAS_RES ? 1 : 3;      // A tiles issued while the last W blocks are still being read
+    static_assert(KS % (FD + 1) == 0, "the fragment ring keeps its phase from tile to tile");
+    static_assert(EARLY <= PA && 2 * NL <= KS, "prologue / direct loads inside the K loop");
     constexpr int OFF_R = DA * TILE;
-    constexpr int OFF_B = 6 * TILE;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -166,68 +177,92 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
     if (nt == 0) return;
 
+    const int M32 = (int)M;
     const int tid = threadIdx.x, lane = tid & 63;
     VT_WS_STAMP(0);
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lg = lane >> 5;
     const int col0 = g * BN + w * STRIP;             // first output column of this wave
 
+    // ---- constant MFMA operands
+    // bias: one more K step whose W-side fragment holds bias[col] at k = 0 and whose A-side fragment is 1 at k = 0;
+    // residual: K steps whose W-side fragment is a 16-column slice of the identity and whose A-side fragments are
+    // read from the residual tile like fragments of A.  bf16 x 1 is exact, so the sum is (A W^T + bias) + residual,
+    // each rounded once in fp32, as with separate additions.
+    uint32_t wb[NB];
+    u32x4 eye[2];
+    {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            wb[j] = 0u;
+            if constexpr (HAS_BIAS) wb[j] = lg == 0 ? (uint32_t)bias[col0 + j * 32 + lr] : 0u;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            eye[h] = z;
+            if constexpr (HAS_RES) {
+                // element e of lane (lr, lg) is k = 8*lg + e of W-side row lr: 1 where 16*h + k == lr
+                const bool mine = (lr >> 4) == h && lg == ((lr & 15) >> 3);
+                const uint32_t one = 0x3f80u << (16 * (lr & 1));
+                const int wd = (lr & 7) >> 1;
+                eye[h].x = mine && wd == 0 ? one : 0u;
+                eye[h].y = mine && wd == 1 ? one : 0u;
+                eye[h].z = mine && wd == 2 ? one : 0u;
+                eye[h].w = mine && wd == 3 ? one : 0u;
+            }
+        }
+    }
+
     // ---- per-lane constants
-    // fragment reads: row lr of the tile, 16-byte chunk (2c + lg) of a 128-byte slab, slot-swizzled
+    // fragment reads: row lr of the tile, 16-byte chunk (2c + lg) of a 128-byte slab, slot-swizzled; cs[c] = cs[0] ^ 32c
     int cs[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) cs[c] = lr * 128 + (((2 * c + lg) ^ ((lr >> 1) & 7)) * 16);
-    // direct loads of a 32-row operand tile (A or a W block): instruction i = w*NL + ii covers slab i/4 and rows
+    // direct loads of a 32-row tile (A, a W block, the residual): instruction i = w*NL + ii covers slab i/4 and rows
     // (i%4)*8 + lane/8; the lane fetches chunk (lane%8) ^ ((row/2)%8) = ((lane%8) ^ (lane/16)) ^ 4*(i%2).
-    // Everything that depends on i is wave-uniform, so two lane constants serve all of a wave's loads.
+    // Everything that depends on i is wave-uniform: byte offset = uniform part + one of two lane constants.
     const int l8 = lane >> 3;
     const int ax16 = ((lane & 7) ^ (lane >> 4)) * 16;
-    auto a_row = [&](int ii, int l8v) -> int { return ((w * NL + ii) & 3) * 8 + l8v; };
-    auto a_off = [&](int ii, int ax16v) -> int { const int i = w * NL + ii; return (i >> 2) * 128 + (ax16v ^ ((i & 1) * 64)); };
-    // the residual tile: 32 rows x RROW bytes as RROW/256 column groups of [32 rows][256 B]; instruction i covers
-    // group i/8 and rows (i%8)*4 + lane/16; inside a row the sixteen 16-byte chunks are XOR-swizzled with the row,
-    // so the epilogue's reads (16 rows at one column) are conflict free.
-    const int l16 = lane >> 4;
-    const int ry16 = ((lane & 15) ^ (lane >> 4)) * 16;
-    auto r_row = [&](int ii, int l16v) -> int { return ((w * NL + ii) & 7) * 4 + l16v; };
-    auto r_off = [&](int ii, int ry16v) -> int { const int i = w * NL + ii; return g * RROW + (i >> 3) * 256 + (ry16v ^ ((i & 3) * 64)); };
-    // epilogue: lane (lr, lg) handles row lr and the 8-column vector (j, q) = chunk cb + lg, cb = 12*w + 4*j + 2*q
-    const int ebase = lr * 256 + ((lg ^ (lr & 15)) * 16);
-    auto e_roff = [&](int j, int q) -> int { const int cb = w * (STRIP / 8) + j * 4 + q * 2; return (cb >> 4) * 8192 + (ebase ^ ((cb & 15) * 16)); };
-    const int lg16 = lg * 16;
-
-    const int M32 = (int)M;
     const uint32_t lda2 = (uint32_t)lda * 2, ldr2 = (uint32_t)ldr * 2, ldo2 = (uint32_t)ldo * 2;   // row pitches, bytes
-    auto tile_row0 = [&](int k) -> int { return (p + k * P) * 32; };
-
-    // tally of vector-memory operations issued by this wave and, per A tile, the tally right after its loads
-    int issued = 0;
-    uint64_t marks = 0;
-    auto issue_a = [&](int k) {
-        const int m0 = tile_row0(k);
-        const uint32_t dst = lds0 + (k % DA) * TILE + w * NL * 1024;
-        const int l8v = fresh(l8), ax16v = fresh(ax16);
-#pragma unroll
-        for (int ii = 0; ii < NL; ii++) {
-            int gm = m0 + a_row(ii, l8v);
-            gm = gm < M32 ? gm : M32 - 1;
-            dma16(A, (uint32_t)gm * lda2 + a_off(ii, ax16v), dst + ii * 1024);
-        }
-        issued += NL;
-        const int sh = (k & 7) * 8;
-        marks = (marks & ~(0xffull << sh)) | ((uint64_t)(issued & 0xff) << sh);
+    const uint32_t va[2] = {l8 * lda2 + ax16, l8 * lda2 + (ax16 ^ 64)};
+    const uint32_t vr[2] = {l8 * ldr2 + ax16, l8 * ldr2 + (ax16 ^ 64)};
+    // First row of this workgroup's k-th tile.  The last tile of the matrix is moved back so that it ends at row M
+    // (its first rows repeat rows of the tile before, recomputed bit for bit), so no tile but a lone first one
+    // (M < 32) reaches past the end.
+    const int m_last = M32 > 32 ? M32 - 32 : 0;
+    auto tile_row0 = [&](int k) -> int { const int m = (p + k * P) * 32; return m < m_last ? m : m_last; };
+    // one direct load of tile rows m0.. from `base` (row pitch `pitch`, `col` bytes into the row) to LDS `dst`;
+    // ii = which of the wave's NL loads, par = ii % 2
+    auto tile_dma = [&](const void *base, uint32_t pitch, uint32_t col, const uint32_t (&v)[2], int m0, int ii, int par,
+                        uint32_t dst) {
+        const int i = w * NL + ii;
+        dma16(base, (uint32_t)(m0 + (i & 3) * 8) * pitch + col + (i >> 2) * 128 + v[par], dst + i * 1024);
     };
-    auto issue_r = [&](int k) {
-        const int m0 = tile_row0(k);
-        const uint32_t dst = lds0 + OFF_R + (k % DR) * TILE + w * NL * 1024;
-        const int l16v = fresh(l16), ry16v = fresh(ry16);
+    // the same for a lone tile of fewer than 32 rows: rows past the end are clamped to the last one
+    auto tile_dma_short = [&](const void *base, uint32_t pitch, uint32_t col, int ii, uint32_t dst) {
+        const int i = w * NL + ii;
+        int gm = (i & 3) * 8 + l8;
+        gm = gm < M32 ? gm : M32 - 1;
+        dma16(base, (uint32_t)gm * pitch + col + (i >> 2) * 128 + (ax16 ^ ((i & 1) * 64)), dst + i * 1024);
+    };
+
+    // tally of vector-memory operations issued by this wave and, per tile, the tally right after its loads
+    int issued = 0;
+    uint64_t marks_a = 0, marks_r = 0;
+    auto set_mark = [](uint64_t &m, int k, int v) {
+        const int sh = (k & 7) * 8;
+        m = (m & ~(0xffull << sh)) | ((uint64_t)(v & 0xff) << sh);
+    };
+    auto after_mark = [&](uint64_t m, int k) -> int { return (issued - (int)((m >> ((k & 7) * 8)) & 0xff)) & 0xff; };
+    auto issue_a_all = [&](int k) {      // prologue only; inside the K loop the six loads are spread out
 #pragma unroll
         for (int ii = 0; ii < NL; ii++) {
-            int gm = m0 + r_row(ii, l16v);
-            gm = gm < M32 ? gm : M32 - 1;
-            dma16(res, (uint32_t)gm * ldr2 + r_off(ii, ry16v), dst + ii * 1024);
+            if (M32 >= 32) tile_dma(A, lda2, 0, va, tile_row0(k), ii, ii & 1, lds0 + (k % DA) * TILE);
+            else tile_dma_short(A, lda2, 0, ii, lds0 + (k % DA) * TILE);
         }
         issued += NL;
+        set_mark(marks_a, k, issued);
     };
 
     // ---- the stationary operand: 12 blocks of 32 W rows (block = 3 * wave + j) pass through the six LDS slots,
@@ -240,7 +275,10 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                 const uint32_t src = (uint32_t)(g * BN + (round * 3 + b) * 32) * KB;
                 const uint32_t dst = lds0 + ((round & 1) * 3 + b) * TILE + w * NL * 1024;
 #pragma unroll
-                for (int ii = 0; ii < NL; ii++) dma16(Wt, src + a_row(ii, l8) * KB + a_off(ii, ax16), dst + ii * 1024);
+                for (int ii = 0; ii < NL; ii++) {
+                    const int i = w * NL + ii;
+                    dma16(Wt, src + ((i & 3) * 8 + l8) * KB + (i >> 2) * 128 + (ax16 ^ ((i & 1) * 64)), dst + ii * 1024);
+                }
             }
         };
         auto read_w = [&](int round) {
@@ -254,14 +292,6 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                     else wfv[j][s - KA] = v;
                 }
         };
-        if constexpr (HAS_BIAS) {
-            // the strip's bias: one direct load by wave 0, the oldest operation of all (lanes past the strip re-read
-            // its last chunk; the LDS area is a full 1 KB)
-            if (w == 0) {
-                const int c = lane < BN / 8 ? lane : BN / 8 - 1;
-                dma16(bias, (uint32_t)(g * BN * 2 + c * 16), lds0 + OFF_B);
-            }
-        }
         issue_w(0);
         issue_w(1);
 #pragma unroll
@@ -269,6 +299,12 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
             if (round < 3) wait_vmcnt<3 * NL>();   // everything but the youngest round has landed
             else wait_vmcnt_dyn(issued);           // ... but the first A tiles
             __syncthreads();
+            if (round == 0) {
+                // the bias values are consumed here as far as the compiler is concerned: their loads are issued
+                // above and waited for now, not next to their first real use in the middle of the pipeline
+#pragma unroll
+                for (int j = 0; j < NB; j++) asm volatile("" : "+v"(wb[j]));
+            }
             if (w == round) read_w(round);
             __syncthreads();                       // the three slots are free again
             if (round + 2 < 4) issue_w(round + 2);
@@ -276,71 +312,53 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                 // slots 0..2 have seen their last W block: the first A tiles can follow
 #pragma unroll
                 for (int k = 0; k < EARLY; k++)
-                    if (k < nt) issue_a(k);
+                    if (k < nt) issue_a_all(k);
             }
         }
     }
     VT_WS_STAMP(1);
+    // ---- rest of the prologue: first residual tiles, remaining first tiles of A
+    if constexpr (HAS_RES) {
+#pragma unroll
+        for (int k = 0; k < PR; k++) {
+            if (k < nt) {
+#pragma unroll
+                for (int ii = 0; ii < NL; ii++) {
+                    if (M32 >= 32) tile_dma(res, ldr2, g * KB, vr, tile_row0(k), ii, ii & 1, lds0 + OFF_R + k * TILE);
+                    else tile_dma_short(res, ldr2, g * KB, ii, lds0 + OFF_R + k * TILE);
+                }
+                issued += NL;
+                set_mark(marks_r, k, issued);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = EARLY; k < PA; k++)
+        if (k < nt) issue_a_all(k);
 
     f32x16 acc[2][NB];
+    u32x4 fa[FD + 1];
 
     // ---- epilogue of one tile, in NU units.  Unit n = 4 * (2j + q) + e turns the accumulator pair
     // (8q + e, 8q + 4 + e) of block j into elements e and 4 + e of the lane's 8-column vector (j, q).
-    // Bias and residual of a vector come from LDS.  The residual (used last in a unit) is fetched right after the
-    // previous vector is stored; so is the bias when it is added last too (no activation) or when registers are
-    // short (activation + residual); otherwise the bias is fetched one unit ahead into a second register set.
-    constexpr bool LATE_BIAS = ACT == VTDGE_ACT_NONE || HAS_RES;
-    constexpr bool BIAS_LAST = ACT == VTDGE_ACT_NONE;
-    u32x4 e_bias, e_res, n_bias;
     uint32_t e_w[4];        // packed pairs of the current vector
     float h0, h1;           // elements of an even unit waiting for their odd neighbours
     EpiUnit un;
-    auto fetch_bias = [&](u32x4 &dst, int vec) {
-        dst = *reinterpret_cast<const u32x4 *>(smem + OFF_B + (w * (STRIP / 8) + (vec / 2) * 4 + (vec % 2) * 2) * 16 + lg16);
-    };
-    auto fetch_res = [&](int k, int vec) {
-        e_res = *reinterpret_cast<const u32x4 *>(smem + OFF_R + (k % DR) * TILE + e_roff(vec / 2, vec % 2));
-    };
-    auto epi_begin = [&](int k) {     // LDS reads for vector 0 of tile k
-        if constexpr (HAS_BIAS) fetch_bias(LATE_BIAS ? e_bias : n_bias, 0);
-        if constexpr (HAS_RES) fetch_res(k, 0);
-    };
-    auto word_lo_hi = [](const u32x4 &v, int e) -> float {   // element e (0..7) of a vector of 8 bf16
-        const uint32_t wd = v[e / 2];
-        return (e & 1) ? bf16hi(wd) : bf16lo(wd);
-    };
-    // part 1 of unit n: out of the accumulator, bias, first third of the activation
     auto epi_part1 = [&](auto pp_tag, int n) {
         constexpr int PP = decltype(pp_tag)::value;
         const int j = n / 8, q = (n / 4) % 2, e = n % 4;
-        if constexpr (HAS_BIAS && !LATE_BIAS) {
-            if (e == 0) e_bias = n_bias;
-        }
         auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[PP][j][8 * q + e]),
                                                   __float_as_uint(acc[PP][j][8 * q + 4 + e]), false, false);
         un.f0 = __uint_as_float(r[0]);
         un.f1 = __uint_as_float(r[1]);
-        if constexpr (HAS_BIAS && !BIAS_LAST) {
-            un.f0 += word_lo_hi(e_bias, e);
-            un.f1 += word_lo_hi(e_bias, 4 + e);
-        }
         if constexpr (ACT == VTDGE_ACT_GELU) gelu_part1(un);
     };
     auto epi_part2 = [&](int n) {
         if constexpr (ACT == VTDGE_ACT_GELU) gelu_part2(un);
     };
-    // part 3: rest of the activation, residual; odd units pack, the fourth unit of a vector stores it
-    auto epi_part3 = [&](int k, int n, unsigned char *orow) {
+    auto epi_part3 = [&](int n, unsigned char *orow) {
         const int j = n / 8, q = (n / 4) % 2, e = n % 4;
         if constexpr (ACT == VTDGE_ACT_GELU) gelu_part3(un);
-        if constexpr (HAS_BIAS && BIAS_LAST) {
-            un.f0 += word_lo_hi(e_bias, e);
-            un.f1 += word_lo_hi(e_bias, 4 + e);
-        }
-        if constexpr (HAS_RES) {
-            un.f0 += word_lo_hi(e_res, e);
-            un.f1 += word_lo_hi(e_res, 4 + e);
-        }
         if (e % 2 == 0) {
             h0 = un.f0;
             h1 = un.f1;
@@ -348,17 +366,10 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
             e_w[e / 2] = pack_bf16x2(h0, un.f0);        // elements e-1, e
             e_w[2 + e / 2] = pack_bf16x2(h1, un.f1);    // elements 4+e-1, 4+e
         }
-        if constexpr (HAS_BIAS && !LATE_BIAS) {
-            if (e == 2 && n + 2 < NU) fetch_bias(n_bias, n / 4 + 1);
-        }
         if (e == 3) {
             u32x4 v;
             v.x = e_w[0]; v.y = e_w[1]; v.z = e_w[2]; v.w = e_w[3];
             *reinterpret_cast<u32x4 *>(orow + (j * 32 + 8 * 2 * q) * 2) = v;
-            if (n + 1 < NU) {
-                if constexpr (HAS_BIAS && LATE_BIAS) fetch_bias(e_bias, n / 4 + 1);
-                if constexpr (HAS_RES) fetch_res(k, n / 4 + 1);
-            }
         }
     };
     auto out_row = [&](int k) -> unsigned char * {
@@ -367,63 +378,142 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         return reinterpret_cast<unsigned char *>(out) + (uint64_t)(uint32_t)gm * ldo2 + (col0 + 8 * lg) * 2;
     };
 
-    // ---- one tile: wait for A(k), multiply into acc[PP]; when EPI, finish tile k-1 (in acc[1-PP]) on the way
+    // wait until this wave's loads of what step k needs have landed: A(k+1) (its first fragments are read at the
+    // end of step k), or A(k) and the residual of tile k
+    auto wait_step = [&](int k) {
+        int after = 255;
+        if constexpr (XT) {
+            if (k + 1 < nt) after = after_mark(marks_a, k + 1);
+        } else {
+            after = after_mark(marks_a, k);
+        }
+        if constexpr (HAS_RES) {
+            const int ar = after_mark(marks_r, k);
+            after = ar < after ? ar : after;
+        }
+        if (after != 255) wait_vmcnt_dyn(after);
+    };
+
+    // ---- one tile: multiplies A(k) into acc[PP]; when EPI, finishes tile k-1 (in acc[1-PP]) on the way.
     auto tile_step = [&](auto pp_tag, auto epi_tag, int k) {
         constexpr int PP = decltype(pp_tag)::value;
         constexpr bool EPI = decltype(epi_tag)::value;
         using PQ = std::integral_constant<int, 1 - PP>;
-        const int after = (issued - (int)((marks >> ((k & 7) * 8)) & 0xff)) & 0xff;
+        const bool more = k + 1 < nt;
         VT_WS_STAMP(3 + 2 * k);
-        wait_vmcnt_dyn(after);
+        wait_step(k);
         VT_WS_STAMP(4 + 2 * k);
-        block_barrier();   // A(k) (and the residual of k-1) are in LDS for every wave; the slots read last step are free
-        if constexpr (HAS_RES) {
-            if (k + 1 < nt) issue_r(k + 1);
-        }
-        if (k + PA < nt) issue_a(k + PA);
+        block_barrier();   // what was awaited is in LDS for every wave; the slots read last step are free
 
-        const unsigned char *at = smem + (k % DA) * TILE;
-        unsigned char *orow = nullptr;
-        if constexpr (EPI) {
-            orow = out_row(k - 1);
-            epi_begin(k - 1);
+        // Direct loads of this step: the residual of tile k+PR and A(k+PA), six each per wave.  The waves take turns
+        // (wave w issues in substeps 6w .. 6w+5: load number s of each tile in substep s, the residual's first), so
+        // the loads of different waves do not queue behind each other at the address unit.  Stores (when EPI) follow
+        // the MFMAs of substeps 3, 7, .., 23.  The tallies count, for this wave, what is issued up to the last load
+        // of each tile.
+        const bool has_a = k + PA < nt;
+        const bool has_r = HAS_RES && k + PR < nt;
+        const int w6 = w * NL;
+        const uint32_t mask_a = has_a ? 0x3fu << w6 : 0u, mask_r = has_r ? 0x3fu << w6 : 0u;
+        {
+            const int start = issued, n = (has_a ? 1 : 0) + (has_r ? 1 : 0);
+            const int st = EPI ? (w6 + 1) / 4 + 1 : 0;        // stores before the loads of substep 6w+5
+            if (has_r) set_mark(marks_r, k + PR, start + (NL - 1) * n + 1 + st);
+            if (has_a) set_mark(marks_a, k + PA, start + NL * n + st);
+            issued = start + NL * n + (EPI ? NB * 2 : 0);
         }
-        // fragments of A are read FD substeps ahead of the MFMAs that use them
-        constexpr int FD = HAS_RES ? 2 : 3;
-        u32x4 fa[FD + 1];
+        const uint32_t dst_a = lds0 + ((k + PA) % DA) * TILE, dst_r = lds0 + OFF_R + ((k + PR) % DR) * TILE;
+        const uint32_t sa = (uint32_t)tile_row0(k + PA) * lda2, sr = (uint32_t)tile_row0(k + PR) * ldr2 + g * KB;
+        auto step_dma = [&](int s) {      // s is a compile-time constant at every call
+            if constexpr (HAS_RES) {
+                if ((mask_r >> s) & 1) dma16(res, sr + (s & 3) * 8 * ldr2 + (s >> 2) * 128 + vr[s & 1], dst_r + s * 1024);
+            }
+            if ((mask_a >> s) & 1) dma16(A, sa + (s & 3) * 8 * lda2 + (s >> 2) * 128 + va[s & 1], dst_a + s * 1024);
+        };
+
+        // fragment addresses of this step: only cs[0] is kept between steps
+        const int cs0 = fresh(cs[0]);
+        const int csl[4] = {cs0, cs0 ^ 32, cs0 ^ 64, cs0 ^ 96};
+        const unsigned char *at = smem + (k % DA) * TILE;
+        const unsigned char *an = smem + ((k + 1) % DA) * TILE;
+        unsigned char *orow = nullptr;
+        if constexpr (EPI) orow = out_row(k - 1);
+        // residual fragments: K steps 6w .. 6w+5 of the residual tile, through a ring of four registers sets
+        u32x4 fr[4];
+        auto read_fr = [&](int i) {            // i-th fragment in the order the MFMAs take them
+            const int t = w * 2 * NB + (i % NB) * 2 + i / NB;
+            fr[i % 4] = *reinterpret_cast<const u32x4 *>(smem + OFF_R + (k % DR) * TILE + (t >> 2) * 4096 +
+                                                          (cs0 ^ ((t & 3) * 32)));
+        };
+        if constexpr (!XT) {
 #pragma unroll
-        for (int s = 0; s < FD; s++) fa[s] = *reinterpret_cast<const u32x4 *>(at + (s >> 2) * 4096 + cs[s & 3]);
+            for (int s = 0; s < FD; s++) fa[s] = *reinterpret_cast<const u32x4 *>(at + (s >> 2) * 4096 + csl[s & 3]);
+        }
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-            if (s + FD < KS)
-                fa[(s + FD) % (FD + 1)] =
-                    *reinterpret_cast<const u32x4 *>(at + ((s + FD) >> 2) * 4096 + cs[(s + FD) & 3]);
-            __builtin_amdgcn_sched_barrier(0);   // keep the read ahead of, not next to, its use
             const u32x4 &f = fa[s % (FD + 1)];
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 if (s == 0) mma_az(acc[PP][j], wfa[j][0], f);
                 else if (s < KA) mma_a(acc[PP][j], wfa[j][s], f);
                 else mma_v(acc[PP][j], wfv[j][s - KA], f);
-                if constexpr (EPI) {
-                    // a few vector instructions behind every MFMA: they execute while it runs
-                    if (j == 0) epi_part1(PQ{}, s);
-                    if (j == 1) epi_part2(s);
-                    if (j == 2) epi_part3(k - 1, s, orow);
+                // behind every MFMA a few other instructions, which issue while it runs
+                if (j == 0) {
+                    // the fragment of A for substep s + FD (the next tile's when this one has no more)
+                    if (s + FD < KS)
+                        fa[(s + FD) % (FD + 1)] =
+                            *reinterpret_cast<const u32x4 *>(at + ((s + FD) >> 2) * 4096 + csl[(s + FD) & 3]);
+                    else if (XT && more)
+                        fa[(s + FD) % (FD + 1)] =
+                            *reinterpret_cast<const u32x4 *>(an + ((s + FD - KS) >> 2) * 4096 + csl[(s + FD - KS) & 3]);
+                    if constexpr (HAS_RES) {
+                        if (s >= KS - 2) read_fr(s - (KS - 2));    // the first two residual fragments
+                    }
+                    if constexpr (EPI) epi_part1(PQ{}, s);
+                }
+                if (j == 1) {
+                    step_dma(s);
+                    if constexpr (EPI) epi_part2(s);
+                }
+                if (j == 2) {
+                    if constexpr (EPI) {
+                        epi_part3(s, orow);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if constexpr (HAS_BIAS) {
+            const u32x4 ones = {fresh(lane) < 32 ? 0x3f80u : 0u, 0u, 0u, 0u};   // made here: no registers held
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                const u32x4 wbj = {wb[j], 0u, 0u, 0u};
+                mma_v_fresh(acc[PP][j], wbj, ones);
+            }
+        }
+        if constexpr (HAS_RES) {
+            // in the order 0, 2, 4, 1, 3, 5 of K steps, so that consecutive MFMAs go to different accumulators
+            read_fr(2);
+            read_fr(3);
+#pragma unroll
+            for (int i = 0; i < 2 * NB; i++) {
+                const int kk = (i % NB) * 2 + i / NB;
+                __builtin_amdgcn_sched_barrier(0);
+                mma_v(acc[PP][kk / 2], eye[kk % 2], fr[i % 4]);
+                if (i < 2) {
                     __builtin_amdgcn_sched_barrier(0);
+                    read_fr(i + 4);
                 }
             }
         }
-        if constexpr (EPI) issued += NB * 2;
     };
 
-    // ---- rest of the prologue: first residual tile (ahead of A(1): a tile's wait covers what was issued before it),
-    // remaining first tiles of A
-    if constexpr (HAS_RES) issue_r(0);
+    if constexpr (XT) {
+        // first tile: its own wait, and its first fragments
+        wait_vmcnt_dyn(after_mark(marks_a, 0));
+        block_barrier();
 #pragma unroll
-    for (int k = EARLY; k < PA; k++)
-        if (k < nt) issue_a(k);
-
+        for (int s = 0; s < FD; s++) fa[s] = *reinterpret_cast<const u32x4 *>(smem + (s >> 2) * 4096 + cs[s & 3]);
+    }
     VT_WS_STAMP(2);
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
@@ -433,38 +523,27 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         tile_step(I1{}, std::true_type{}, k);
         tile_step(I0{}, std::true_type{}, k + 1);
     }
-    if (k < nt) {
-        tile_step(I1{}, std::true_type{}, k);
-        k++;
-    }
+    if (k < nt) tile_step(I1{}, std::true_type{}, k);
     VT_WS_STAMP(3 + 2 * nt);
-    // ---- last tile's epilogue (its residual was fetched two steps ago: wait for everything, publish)
-    wait_vmcnt<0>();
+    // ---- last tile's epilogue
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs' results must have reached the registers
-    block_barrier();
     unsigned char *orow = out_row(nt - 1);
-    epi_begin(nt - 1);
     if ((nt - 1) & 1) {
 #pragma unroll
-        for (int n = 0; n < NU; n++) {
-            epi_part1(I1{}, n);
-            epi_part2(n);
-            epi_part3(nt - 1, n, orow);
-        }
-    } else {
+        for (int j = 0; j < NB; j++) acc[0][j] = acc[1][j];
+    }
 #pragma unroll
-        for (int n = 0; n < NU; n++) {
-            epi_part1(I0{}, n);
-            epi_part2(n);
-            epi_part3(nt - 1, n, orow);
-        }
+    for (int n = 0; n < NU; n++) {
+        epi_part1(I0{}, n);
+        epi_part2(n);
+        epi_part3(n, orow);
     }
     VT_WS_STAMP(4 + 2 * nt);
 }
 
 // ----------------------------------------------------------------------------- host
-bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, const void *bias,
-                          const void *res, const void *out)
+bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
+                          const void *bias, const void *res, const void *out)
 {
     static int off = -1;   // VTDGE_LINEAR_WS=0 keeps these shapes on the streaming kernel (A/B timing)
     if (off < 0) {
@@ -472,9 +551,12 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
         off = (e && atoi(e) == 0) ? 1 : 0;
     }
     if (off) return false;
+    // the residual is added inside the accumulator, i.e. before an activation: such a pair goes elsewhere
+    if (res != nullptr && act != VTDGE_ACT_NONE) return false;
     return esz == 2 && K == 384 && lda < (1ll << 31) && ldo < (1ll << 31) && ldr < (1ll << 31) && N % 384 == 0 &&
-           N / 384 <= 8 && rows >= 2048 && rows * lda < (1ll << 31) && (res == nullptr || rows * ldr < (1ll << 31)) && lda % 8 == 0 && ldo % 8 == 0 &&
-           (res == nullptr || ldr % 8 == 0) && (((uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15) == 0;
+           N / 384 <= 8 && rows >= 2048 && rows * lda < (1ll << 31) && (res == nullptr || rows * ldr < (1ll << 31)) &&
+           lda % 8 == 0 && ldo % 8 == 0 && (res == nullptr || ldr % 8 == 0) &&
+           (((uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15) == 0;
 }
 
 template <int ACT, bool HB, bool HR>
@@ -482,7 +564,7 @@ static int go_ws(const void *A, int64_t lda, const void *W, const void *bias, co
                  int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
 {
     constexpr int KS = 24, NB = 3;
-    constexpr size_t lds = (size_t)6 * 32 * KS * 32 + 1024;   // six 32-row tiles + the strip's bias
+    constexpr size_t lds = (size_t)6 * 32 * KS * 32;   // six 32-row tiles
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR>;
     static bool attr_done = false;  // one flag per instantiation
@@ -512,9 +594,11 @@ int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias
     const bool hb = bias != nullptr, hr = res != nullptr;
 #define VT_WS(ACT, HB, HR) return go_ws<ACT, HB, HR>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st)
     if (act == VTDGE_ACT_GELU) {
-        if (hb && hr) VT_WS(VTDGE_ACT_GELU, true, true);
+        if (hr) {
+            set_error("linear: activation with residual is not built in the weight-stationary kernel");
+            return VTDGE_ERR_UNSUPPORTED;
+        }
         if (hb) VT_WS(VTDGE_ACT_GELU, true, false);
-        if (hr) VT_WS(VTDGE_ACT_GELU, false, true);
         VT_WS(VTDGE_ACT_GELU, false, false);
     }
     if (hb && hr) VT_WS(VTDGE_ACT_NONE, true, true);
