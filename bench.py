@@ -82,13 +82,14 @@ def kernel_symbol(name, tag, dt, n_keys=0):
     if name == "vtdge_decompress":
         return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
     if name == "vtdge_layernorm":
-        return f"layernorm_kernel<{T}, {gs(tag[3])}>"
+        nv = tag[3] * esz // 16                           # 16-byte vectors per row
+        return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
     if name == "vtdge_sparse_attention":
         if dt == "bf16" and tag[3] == 64:
             return "sparse_attention_bf16_d64_resident_kernel" if tag[4] <= 288 else "sparse_attention_bf16_d64_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
-        return f"router_kernel<{T}, {gs(tag[1])}>"
+        return f"router_kernel<{T}, 4, {gs(tag[1])}>"     # region size 4 in every model of these workloads
     if name == "vtdge_index_to_patch":
         return "patch_count_scan_kernel+patch_write_kernel"
     return name

@@ -80,21 +80,27 @@ __device__ __forceinline__ void mma_az(f32x16 &d, const u32x4 &wfrag, const u32x
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "a"(wfrag), "v"(afrag));
 }
 
-// s_waitcnt vmcnt(n) for a wave-uniform runtime n (a multiple of 6; more than 60 waits for 60)
+// s_waitcnt vmcnt(n) for a wave-uniform runtime n, rounded down to a multiple of 6 and to at most 42 (waiting for
+// fewer operations in flight than allowed is always safe).  A balanced tree of three compares: the immediate of
+// s_waitcnt cannot come from a register.
 __device__ __forceinline__ void wait_vmcnt_dyn(int n)
 {
-    switch (n / 6) {
-    case 0: wait_vmcnt<0>(); break;
-    case 1: wait_vmcnt<6>(); break;
-    case 2: wait_vmcnt<12>(); break;
-    case 3: wait_vmcnt<18>(); break;
-    case 4: wait_vmcnt<24>(); break;
-    case 5: wait_vmcnt<30>(); break;
-    case 6: wait_vmcnt<36>(); break;
-    case 7: wait_vmcnt<42>(); break;
-    case 8: wait_vmcnt<48>(); break;
-    case 9: wait_vmcnt<54>(); break;
-    default: wait_vmcnt<60>(); break;
+    if (n >= 24) {
+        if (n >= 36) {
+            if (n >= 42) wait_vmcnt<42>();
+            else wait_vmcnt<36>();
+        } else {
+            if (n >= 30) wait_vmcnt<30>();
+            else wait_vmcnt<24>();
+        }
+    } else {
+        if (n >= 12) {
+            if (n >= 18) wait_vmcnt<18>();
+            else wait_vmcnt<12>();
+        } else {
+            if (n >= 6) wait_vmcnt<6>();
+            else wait_vmcnt<0>();
+        }
     }
 }
 
@@ -146,7 +152,8 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
     constexpr int STRIP = NB * 32;              // output columns per wave
     constexpr int BN = 4 * STRIP;               // output columns per workgroup
-    constexpr int DA = HAS_RES ? 3 : 6;         // A ring depth (tiles); the residual ring takes the other three slots
+    constexpr int DA = HAS_RES ? 3 : 4;         // A ring depth (tiles): deeper gains nothing and lengthens the start;
+                                                // behind a residual its ring takes three of the six slots
     constexpr int DR = 3;
     constexpr int PA = DA - 1;                  // step k issues the loads of A(k + PA)
     constexpr int PR = DR - 1;                  // ... and of the residual of tile k + PR
@@ -157,7 +164,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     constexpr int NU = NB * 8;                  // epilogue units per tile (two elements each)
     constexpr int KA = KS - 3;                  // substeps whose W fragments live in accumulation registers
     constexpr int FD = (HAS_RES || ACT != VTDGE_ACT_NONE) ? 2 : 3;         // fragments of A are read FD substeps ahead of their MFMAs
-    constexpr int EARLY = PA < 3 ? PA : 3;      // A tiles issued while the last W blocks are still being read
+    constexpr int EARLY = 2;                    // A tiles issued while the last W blocks are still being read
     static_assert(KS % 4 == 0 && NL * 4 * 1024 == TILE && BN * 2 == KB, "tile geometry (residual rows = A rows)");
     static_assert(!(HAS_RES && ACT != VTDGE_ACT_NONE), "the residual is summed in the accumulator, ahead of an activation");
     static_assert(NL == 6 && NB == 3, "the vmcnt bookkeeping counts in units of 6");
@@ -265,56 +272,73 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         set_mark(marks_a, k, issued);
     };
 
-    // ---- the stationary operand: 12 blocks of 32 W rows (block = 3 * wave + j) pass through the six LDS slots,
-    // three at a time; wave `r` picks its fragments out of round r.
+    // ---- the stationary operand: 12 blocks of 32 W rows (block 3 * wave + j holds wave's j-th column block) pass
+    // through the six LDS slots.  Round j brings every wave its j-th block, so all four waves read at once; the
+    // loads of the next round are in flight meanwhile (slots: round 0 -> 0..3; round 1 -> 4, 5, 0, 1;
+    // round 2 -> 2, 3, 4, 5), and the first two tiles of A follow into slots 0 and 1 as soon as those are free.
     u32x4 wfa[NB][KA], wfv[NB][KS - KA];
     {
-        auto issue_w = [&](int round) {   // blocks 3*round .. 3*round+2 -> slots 3*(round&1) ..
+        // Every workgroup of a column group reads the same 288 KB, and the workgroups of an XCD would walk them in
+        // step, all on the same few L2 channels at any moment: each starts its walk somewhere else.
+        const int rot = slot % NL, rot4 = (slot / NL) & 3;
+        auto issue_w = [&](int wave, int j, int lds_slot) {   // this wave's share (NL loads) of block (wave, j)
+            const uint32_t src = (uint32_t)(g * BN + (wave * NB + j) * 32) * KB;
+            const uint32_t dst = lds0 + lds_slot * TILE;
 #pragma unroll
-            for (int b = 0; b < 3; b++) {
-                const uint32_t src = (uint32_t)(g * BN + (round * 3 + b) * 32) * KB;
-                const uint32_t dst = lds0 + ((round & 1) * 3 + b) * TILE + w * NL * 1024;
-#pragma unroll
-                for (int ii = 0; ii < NL; ii++) {
-                    const int i = w * NL + ii;
-                    dma16(Wt, src + ((i & 3) * 8 + l8) * KB + (i >> 2) * 128 + (ax16 ^ ((i & 1) * 64)), dst + ii * 1024);
-                }
+            for (int ii = 0; ii < NL; ii++) {
+                int i2 = ii + rot;
+                i2 = i2 >= NL ? i2 - NL : i2;
+                const int i = w * NL + i2;
+                dma16(Wt, src + ((i & 3) * 8 + l8) * KB + (i >> 2) * 128 + (ax16 ^ ((i & 1) * 64)), dst + i * 1024);
             }
         };
-        auto read_w = [&](int round) {
-            const unsigned char *base = smem + (round & 1) * 3 * TILE;
+        auto read_w = [&](int j, int slot) {
+            const unsigned char *base = smem + slot * TILE;
 #pragma unroll
-            for (int j = 0; j < NB; j++)
-#pragma unroll
-                for (int s = 0; s < KS; s++) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(base + j * TILE + (s >> 2) * 4096 + cs[s & 3]);
-                    if (s < KA) wfa[j][s] = v;
-                    else wfv[j][s - KA] = v;
-                }
+            for (int s = 0; s < KS; s++) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(base + (s >> 2) * 4096 + cs[s & 3]);
+                if (s < KA) wfa[j][s] = v;
+                else wfv[j][s - KA] = v;
+            }
         };
-        issue_w(0);
-        issue_w(1);
 #pragma unroll
-        for (int round = 0; round < 4; round++) {
-            if (round < 3) wait_vmcnt<3 * NL>();   // everything but the youngest round has landed
-            else wait_vmcnt_dyn(issued);           // ... but the first A tiles
-            __syncthreads();
-            if (round == 0) {
-                // the bias values are consumed here as far as the compiler is concerned: their loads are issued
-                // above and waited for now, not next to their first real use in the middle of the pipeline
+        for (int v = 0; v < 4; v++) issue_w((v + rot4) & 3, 0, (v + rot4) & 3);
+        issue_w(0, 1, 4);
+        issue_w(1, 1, 5);
+        VT_WS_STAMP(40);
+        wait_vmcnt<2 * NL>();                  // round 0 has landed
+        VT_WS_STAMP(41);
+        __syncthreads();
+        // the bias values are consumed here as far as the compiler is concerned: their loads are issued above and
+        // waited for now, not next to their first real use in the middle of the pipeline
 #pragma unroll
-                for (int j = 0; j < NB; j++) asm volatile("" : "+v"(wb[j]));
-            }
-            if (w == round) read_w(round);
-            __syncthreads();                       // the three slots are free again
-            if (round + 2 < 4) issue_w(round + 2);
-            if (round == 2) {
-                // slots 0..2 have seen their last W block: the first A tiles can follow
+        for (int j = 0; j < NB; j++) asm volatile("" : "+v"(wb[j]));
+        read_w(0, w);
+        VT_WS_STAMP(42);
+        __syncthreads();                       // slots 0..3 are free
+        issue_w(2, 1, 0);
+        issue_w(3, 1, 1);
+        issue_w(0, 2, 2);
+        issue_w(1, 2, 3);
+        VT_WS_STAMP(43);
+        wait_vmcnt<2 * NL>();                  // round 1 has landed
+        VT_WS_STAMP(44);
+        __syncthreads();
+        read_w(1, w < 2 ? 4 + w : w - 2);
+        VT_WS_STAMP(45);
+        __syncthreads();                       // slots 4, 5, 0, 1 are free
+        issue_w(2, 2, 4);
+        issue_w(3, 2, 5);
 #pragma unroll
-                for (int k = 0; k < EARLY; k++)
-                    if (k < nt) issue_a_all(k);
-            }
-        }
+        for (int k = 0; k < EARLY; k++)
+            if (k < nt) issue_a_all(k);
+        VT_WS_STAMP(46);
+        wait_vmcnt_dyn(issued);                // round 2 has landed (all but the tiles of A)
+        VT_WS_STAMP(47);
+        __syncthreads();
+        read_w(2, 2 + w);
+        VT_WS_STAMP(48);
+        __syncthreads();                       // slots 2..5 are free
     }
     VT_WS_STAMP(1);
     // ---- rest of the prologue: first residual tiles, remaining first tiles of A
