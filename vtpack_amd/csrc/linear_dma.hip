@@ -59,14 +59,17 @@ template <> __device__ __forceinline__ float gelu_fn<bf16_t>(float v)
 // inside an XCD the (m-tile, n-tile) pairs are walked n-fastest, so the n-tiles sharing an A tile run
 // concurrently on CUs that share an L2.  The mapping does not depend on the live row count, which only
 // trims each XCD's list.
-template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HAS_BIAS, bool HAS_RES>
+// NSTAGE = depth of the operand ring (3, or 2 for tiles whose stages are too large for three); LATE = fetch bias and
+// residual in the epilogue itself instead of during the last stage (large wave tiles have no registers to park them).
+template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HAS_BIAS, bool HAS_RES, int NSTAGE = 3,
+          bool LATE = false>
 __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
     const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, const T *__restrict__ bias,
     const T *__restrict__ res, int64_t ldr, T *__restrict__ out, int64_t ldo, const int64_t *__restrict__ rows_dev,
     int64_t rows, int N, int K)
 {
     constexpr int ESZ = sizeof(T);
-    constexpr int NSTAGE = 3;
+    static_assert(NSTAGE == 2 || NSTAGE == 3, "ring depth");
     constexpr int NWC = WGM * WGN;                   // MFMA waves
     constexpr int TM = BM / WGM, TN = BN / WGN;      // wave tile
     constexpr int IM = TM / 32, JN = TN / 32;        // 32x32 MFMA blocks per wave
@@ -127,14 +130,16 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                 if (++it_tile < nt) set_tile(it_tile);
             }
         };
-        if (issued < G) issue_next();
-        if (issued < G) issue_next();
+#pragma unroll
+        for (int i = 0; i < NSTAGE - 1; i++)
+            if (issued < G) issue_next();
         for (int g = 0; g < G; g++) {
-            // stage g has landed once at most the NLW loads of stage g+1 are outstanding (loads retire in order)
-            if (g + 1 < G) wait_vmcnt<NLW>();
+            // stage g has landed once at most the loads of the younger stages in flight are outstanding (loads
+            // retire in order)
+            if (g + NSTAGE - 2 < G) wait_vmcnt<(NSTAGE - 2) * NLW>();
             else wait_vmcnt<0>();
             block_barrier();                         // stage g visible to the MFMA waves; slot of g-1 is free
-            if (issued < G) issue_next();            // stage g+2
+            if (issued < G) issue_next();            // stage g + NSTAGE - 1
         }
         return;
     }
@@ -168,7 +173,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
         const int u = wg + tk * nwg;
         const int64_t m0 = (int64_t)((u / tiles_n) * 8 + xcd) * BM;
         const int n0 = (u % tiles_n) * BN;
-        if (last) {
+        if (last && !LATE) {
             // issue the epilogue's reads now; they return while the last stage is multiplied
 #pragma unroll
             for (int j = 0; j < JN; j++)
@@ -231,6 +236,15 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                         for (int e = 0; e < 4; e++) f[e] = acc[i][j][4 * q + e];
                         col = n0 + wn * TN + j * 32 + 8 * q + 4 * lg;
                     }
+                    if constexpr (LATE) {
+                        const u32x4 z = {0u, 0u, 0u, 0u};
+                        braw[j][q] = z;
+                        rraw[i][j][q] = z;
+                        if constexpr (HAS_BIAS)
+                            if (col < N) braw[j][q] = *reinterpret_cast<const u32x4 *>(bias + col);
+                        if constexpr (HAS_RES)
+                            if (row < M && col < N) rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + row * ldr + col);
+                    }
                     if constexpr (HAS_BIAS) {
                         float bv[EPL];
                         Elem<T>::unpack(braw[j][q], bv);
@@ -266,10 +280,12 @@ template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool H
 static int go(const LinArgs &a)
 {
     constexpr int NW = WGM * WGN + NWP;
-    constexpr size_t lds = (size_t)3 * (BM + BN) * DKB;
+    constexpr int NSTAGE = (size_t)3 * (BM + BN) * DKB <= 160 * 1024 ? 3 : 2;
+    constexpr bool LATE = (BM / WGM) * (BN / WGN) > 64 * 64;      // wave tiles beyond 64 x 64
+    constexpr size_t lds = (size_t)NSTAGE * (BM + BN) * DKB;
     static_assert(lds <= 160 * 1024, "LDS budget");
     constexpr int WGS_PER_CU = lds <= 80 * 1024 ? 2 : 1;
-    auto kern = linear_dma_kernel<T, BM, BN, WGM, WGN, NWP, ACT, HB, HR>;
+    auto kern = linear_dma_kernel<T, BM, BN, WGM, WGN, NWP, ACT, HB, HR, NSTAGE, LATE>;
     static bool attr_done = false;  // one flag per instantiation
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -333,6 +349,7 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
     int cfg = tuning_override();
     if (cfg < 0) {
         // wide outputs: 256x128 tiles on 8 MFMA waves; narrow ones (N <= 512): 128x128 on 4, for more tiles
+        // (128x384 tiles, whole rows of a narrow output on a two-stage ring, measured no faster: override 6)
         cfg = N >= 768 ? 0 : 1;
     }
     switch (cfg) {
@@ -341,6 +358,7 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
     case 2: return pick_epilogue<T, 256, 128, 4, 2, 2>(a);
     case 3: return pick_epilogue<T, 256, 128, 2, 2, 4>(a);
     case 4: return pick_epilogue<T, 128, 128, 4, 2, 4>(a);
+    case 6: return pick_epilogue<T, 128, 384, 2, 4, 4>(a);
     default: return pick_epilogue<T, 128, 256, 2, 4, 4>(a);
     }
 }
