@@ -81,6 +81,8 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}>"
     if name == "vtdge_decompress":
         return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
+    if name == "vtdge_decompress_layernorm":
+        return f"decompress_ln_kernel<{T}, {b(tag[1])}, {gs(tag[2])}>"
     if name == "vtdge_layernorm":
         nv = tag[3] * esz // 16                           # 16-byte vectors per row
         return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
@@ -91,7 +93,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
     if name == "vtdge_router":
         return f"router_kernel<{T}, 4, {gs(tag[1])}>"     # region size 4 in every model of these workloads
     if name == "vtdge_index_to_patch":
-        return "patch_count_scan_kernel+patch_write_kernel"
+        return "patch_write_kernel<true>"      # one launch for batch * regions <= 16384 (all workloads here)
     return name
 
 
@@ -125,6 +127,9 @@ def algorithmic_work(name, tag, esz, geo):
         return "hbm", B * N * C * esz + 32 * L + L * C * esz * (2 if tag[1] else 1)
     if name == "vtdge_decompress":
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + (2 if tag[2] else 1) * B * N * C * esz
+    if name == "vtdge_decompress_layernorm":
+        # the scatter-back plus one more write of every token (the next block's first LayerNorm)
+        return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + 3 * B * N * C * esz
     if name == "vtdge_layernorm":
         rows = L if tag[1] else tag[2]
         return "hbm", 2.0 * rows * tag[3] * esz

@@ -105,6 +105,16 @@ int vtdge_decompress(const void *in, const void *sub, const int64_t *patches, co
                      int64_t rows, const void *ref, void *out, int B, int N, int C, int W, int extra,
                      int dtype, void *stream);
 
+/* The same scatter with `ref` present, plus the LayerNorm of every token written:
+ *   out[b,t,:] = (in[row,:] - sub[row,:]) + ref[b,t,:],   ln_out[b,t,:] = LayerNorm(out[b,t,:])
+ * i.e. the last step of one block (vtpack/layers/dge.py:87-112) together with the first LayerNorm of the next
+ * (norm1 at vtpack/models/dge/deit_dge.py:127), which would read the same tokens back.  The statistics are taken
+ * from the values as stored in `out`.  Rows of at most 64 16-byte vectors (C <= 512 in bf16, 256 in fp32). */
+int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *patches, const int64_t *rows_dev,
+                               int64_t rows, const void *ref, void *out, void *ln_out, const void *ln_weight,
+                               const void *ln_bias, float ln_eps, int B, int N, int C, int W, int extra, int dtype,
+                               void *stream);
+
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */
 int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out, const int64_t *rows_dev,

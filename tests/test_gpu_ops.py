@@ -30,7 +30,10 @@ def _t(a, dev, dtype=None):
     (33, 4, 4, 1, [2, 1]),
     (7, 4, 4, 1, [1]),
     (2, 20, 20, 1, [4, 2, 1]),    # > 256 regions per sample: several passes of the LDS scan
-    (1500, 4, 4, 1, [4, 2, 1]),   # > 1024 samples: several passes of the sample scan
+    (1500, 4, 4, 1, [4, 2, 1]),   # > 1024 samples: several passes of the sample scan (two-kernel path)
+    (256, 4, 4, 1, [4, 2, 1]),    # the headline batch: one launch, every sample sums the counts before it
+    (64, 8, 8, 1, [4, 2, 1]),
+    (300, 8, 8, 0, [4, 2, 1]),    # 19200 regions: just past the single-launch limit
 ])
 def test_index_to_patch_bit_exact(dev, B, Hr, Wr, extra, splits):
     from vtpack_amd import _C
@@ -114,6 +117,46 @@ def test_decompress_fused_subtract(dev, dtype):
     got = ops.decompress(_t(q, dev, dtype), _t(patches, dev), _t(ref, dev, dtype), W, extra, add_ref=True,
                          sub=_t(comp, dev, dtype))
     assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,W,extra,C", [(4, 16, 16, 1, 192), (2, 32, 32, 1, 384), (3, 8, 12, 0, 64), (2, 8, 8, 2, 256)])
+def test_decompress_with_layernorm(dev, dtype, B, H, W, extra, C):
+    """The scatter-back that also writes the next block's first LayerNorm: `out` is bit for bit the plain
+    scatter-back, and the second output is LayerNorm of `out` as stored."""
+    from vtpack_amd import ops
+    if C * (2 if dtype == torch.bfloat16 else 4) > 1024:
+        pytest.skip("rows longer than 64 vectors go through the separate kernels")
+    idx = random_indices(B + C + 1, B, H // 4, W // 4)
+    patches, _ = orc.index_to_patch(idx, SPLITS, 4, extra)
+    q, comp = randn(C + 4, patches.shape[0], C), randn(C + 5, patches.shape[0], C)
+    ref = randn(C + 6, B, extra + H * W, C)
+    w, b = randn(C + 7, C) * 0.2 + 1, randn(C + 8, C) * 0.1
+    if dtype == torch.bfloat16:
+        q, comp, ref, w, b = bf16_round(q), bf16_round(comp), bf16_round(ref), bf16_round(w), bf16_round(b)
+    delta = torch.from_numpy(q - comp).to(dtype).float().numpy()
+    want = torch.from_numpy(orc.decompress(delta, patches, ref, H, W, extra, True)).to(dtype)
+    want_ln = torch.nn.functional.layer_norm(want.float(), (C,), torch.from_numpy(w), torch.from_numpy(b), 1e-6)
+    got, got_ln = ops.decompress_layernorm(_t(q, dev, dtype), _t(patches, dev), _t(ref, dev, dtype), W, extra,
+                                           _t(w, dev, dtype), _t(b, dev, dtype), 1e-6, sub=_t(comp, dev, dtype))
+    assert torch.equal(got.cpu(), want)
+    assert_close(got_ln.float(), want_ln, dtype, "decompress + layernorm")
+    # the separate LayerNorm kernel on the same tokens gives the same numbers
+    sep = ops.layernorm(got, _t(w, dev, dtype), _t(b, dev, dtype), 1e-6)
+    assert abs_err(got_ln, sep) <= (1e-6 if dtype == torch.float32 else 2 ** -6)
+
+
+def test_decompress_with_layernorm_refuses_long_rows(dev):
+    from vtpack_amd import ops
+    from vtpack_amd._lib import VtdgeError
+    B, H, W, C = 1, 4, 4, 1024
+    patches, _ = orc.index_to_patch(np.zeros((B, 1, 1), dtype=np.int64), SPLITS, 4, 0)
+    z = torch.zeros(patches.shape[0], C, device=dev, dtype=torch.bfloat16)
+    ref = torch.zeros(B, H * W, C, device=dev, dtype=torch.bfloat16)
+    g = torch.ones(C, device=dev, dtype=torch.bfloat16)
+    assert not ops.fits_decompress_layernorm(ref)
+    with pytest.raises(VtdgeError):
+        ops.decompress_layernorm(z, _t(patches, dev), ref, W, 0, g, g, 1e-6)
 
 
 def test_device_side_row_count(dev):

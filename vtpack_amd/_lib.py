@@ -29,6 +29,7 @@ SIGNATURES = {
     "vtdge_index_to_patch_dense": [_p, _i, _i, _i, _i, _i, _i, _p, _p],
     "vtdge_compress": [_p, _p, _p, _l, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_decompress": [_p, _p, _p, _p, _l, _p, _p, _i, _i, _i, _i, _i, _i, _p],
+    "vtdge_decompress_layernorm": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_layernorm": [_p, _p, _p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_linear": [_p, _l, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],
     "vtdge_sparse_attention": [_p, _l, _l, _p, _p, _l, _l, _l, _p, _p, _l, _l, _i, _i, _i, _i, _i, _f, _i, _p],

@@ -150,6 +150,25 @@ __device__ __forceinline__ float wave_sum(float v)
 #undef VT_DPP_ADD
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// The same sum for NV values at once, one step of all of them after the other: NV independent dependency chains
+// instead of NV times one.
+template <int NV> __device__ __forceinline__ void wave_sum_n(float (&v)[NV])
+{
+#define VT_DPP_STEP(ctrl, row_mask)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < NV; i++)                                                           \
+        v[i] += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[i]), ctrl, \
+                                                                      row_mask, 0xf, true))
+    VT_DPP_STEP(0x111, 0xf);
+    VT_DPP_STEP(0x112, 0xf);
+    VT_DPP_STEP(0x114, 0xf);
+    VT_DPP_STEP(0x118, 0xf);
+    VT_DPP_STEP(0x142, 0xa);
+    VT_DPP_STEP(0x143, 0xc);
+#undef VT_DPP_STEP
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+        v[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[i]), 63));
+}
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll

@@ -7,6 +7,7 @@
 // with fully coalesced 16-byte accesses and narrow rows (C = 64, 128: the
 // first PVT stages) still keep every lane of the wavefront busy.
 #include "common.h"
+#include <type_traits>
 
 namespace vtdge {
 
@@ -17,6 +18,17 @@ constexpr int MAX_IT = 3;          // 16-byte vectors per lane: C <= 64*3*VEC
 static int group_size(int nvec) { return nvec > 32 ? 64 : nvec > 16 ? 32 : nvec > 8 ? 16 : 8; }
 
 // sum over the GS lanes of a row's group, returned in each of them
+template <int GS, int NV> __device__ __forceinline__ void group_sum_n(float (&v)[NV])
+{
+    if constexpr (GS == 64) {
+        wave_sum_n<NV>(v);
+    } else {
+#pragma unroll
+        for (int o = GS / 2; o > 0; o >>= 1)
+#pragma unroll
+            for (int i = 0; i < NV; i++) v[i] += __shfl_xor(v[i], o, WAVE);
+    }
+}
 template <int GS> __device__ __forceinline__ float group_sum(float v)
 {
     if constexpr (GS == 64) {
@@ -169,22 +181,45 @@ __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *_
 // Step 2: one workgroup per sample.  The per-region query counts go through an
 // LDS-staged wavefront prefix sum (256 regions per pass); each thread then
 // emits the descriptors of its own region at offsets[b] + extra + prefix.
+//
+// FUSED: the workgroup also finds its own first row, as the sum of the query counts of all samples before it (it
+// reads their gate indices itself: a few KB out of L2 for the batch sizes this variant is launched for), and writes
+// offsets / lengths; no first step then, and no dependency between workgroups.
+template <bool FUSED>
 __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restrict__ indices,
                                                            const int64_t *__restrict__ splits,
-                                                           const int64_t *__restrict__ offsets, int Hr, int Wr,
-                                                           int S, int R, int extra, int64_t *__restrict__ patches,
-                                                           int64_t capacity)
+                                                           int64_t *__restrict__ offsets, int64_t *__restrict__ lengths,
+                                                           int Hr, int Wr, int S, int R, int extra,
+                                                           int64_t *__restrict__ patches, int64_t capacity)
 {
     __shared__ int wave_tot[4];
     __shared__ int carry_s;
     __shared__ int split_s[VTDGE_MAX_SPLITS];
+    __shared__ int64_t before_s[4];
     const int b = blockIdx.x;
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int nreg = Hr * Wr;
     if (threadIdx.x < VTDGE_MAX_SPLITS) split_s[threadIdx.x] = threadIdx.x < S ? (int)splits[threadIdx.x] : 1;
     if (threadIdx.x == 0) carry_s = 0;
     __syncthreads();
-    const int64_t row0 = offsets[b];
+    int64_t row0;
+    if constexpr (FUSED) {
+        int64_t part = 0;
+        for (int64_t i = threadIdx.x; i < (int64_t)b * nreg; i += 256) {
+            int64_t g = indices[i];
+            g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+            const int ps = split_s[g];
+            part += ps * ps;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, WAVE);
+        if (lane == 0) before_s[wid] = part;
+        __syncthreads();
+        row0 = before_s[0] + before_s[1] + before_s[2] + before_s[3] + (int64_t)b * extra;
+        if (threadIdx.x == 0) offsets[b] = row0;
+    } else {
+        row0 = offsets[b];
+    }
     for (int e = threadIdx.x; e < extra; e += 256) {
         const int64_t row = row0 + e;
         if (row < capacity) {
@@ -230,6 +265,13 @@ __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restr
         __syncthreads();
         if (threadIdx.x == 255) carry_s = before + inc;
         __syncthreads();
+    }
+    if constexpr (FUSED) {
+        if (threadIdx.x == 0) {
+            const int64_t len = (int64_t)extra + carry_s;
+            lengths[b] = len;
+            if (b == (int)gridDim.x - 1) offsets[b + 1] = row0 + len;
+        }
     }
 }
 
@@ -466,6 +508,109 @@ __global__ __launch_bounds__(256) void decompress_kernel(const T *__restrict__ i
     }
 }
 
+// Scatter back and LayerNorm in one pass: out = (in - sub) + ref as above, and ln_out = LayerNorm(out) of every
+// token written (what the next block's first LayerNorm would read back and compute).  One group of GS lanes per
+// packed row, one 16-byte vector per lane (rows of at most GS vectors); the tokens of the window are finished one
+// after the other: sum, rounded as it is stored, then two-pass statistics over the group, affine, second store.
+template <typename T, bool SUB, int GS>
+__global__ __launch_bounds__(256) void decompress_ln_kernel(const T *__restrict__ in, const T *__restrict__ sub,
+                                                             const int64_t *__restrict__ patches,
+                                                             const int64_t *__restrict__ rows_dev, int64_t rows,
+                                                             const T *__restrict__ ref, T *__restrict__ out,
+                                                             T *__restrict__ ln_out, const T *__restrict__ ln_w,
+                                                             const T *__restrict__ ln_b, float eps, int N, int C,
+                                                             int W, int extra)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & (GS - 1);
+    const int64_t row = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
+    if (row >= live_rows(rows_dev, rows)) return;
+    const int64_t *p = patches + 4 * row;
+    const int64_t b = p[0], y0 = p[1], x0 = p[2];
+    const int sz = y0 < 0 ? 1 : (int)p[3];
+    const int nvec = C / VEC;
+    const bool act = lane < nvec;
+    const int v = act ? lane : 0;        // idle lanes shadow lane 0's addresses and store nothing
+
+    float d[VEC], w[VEC], bb[VEC];
+    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(in + row * (int64_t)C + v * VEC), d);
+    if constexpr (SUB) {
+        float sv[VEC];
+        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(sub + row * (int64_t)C + v * VEC), sv);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) d[c] = Elem<T>::round(d[c] - sv[c]);
+    }
+    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ln_w + v * VEC), w);
+    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ln_b + v * VEC), bb);
+    const int64_t tok = y0 < 0 ? (-y0 - 1) : (y0 * W + x0 + extra);
+    const int64_t off = (b * N + tok) * (int64_t)C + v * VEC;
+
+    // NT tokens at a time (their reductions interleave): raw = their vectors of ref, o = their element offsets
+    auto finish = [&](auto nt_tag, const u32x4 *raw, const int64_t *o) {
+        constexpr int NT = decltype(nt_tag)::value;
+        float val[NT][VEC], s[NT], q[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float r[VEC];
+            Elem<T>::unpack(raw[t], r);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) r[c] += d[c];
+            const u32x4 packed = Elem<T>::pack(r);
+            if (act) *reinterpret_cast<u32x4 *>(out + o[t]) = packed;
+            Elem<T>::unpack(packed, val[t]);                      // as stored
+            s[t] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) s[t] += act ? val[t][c] : 0.f;
+        }
+        group_sum_n<GS, NT>(s);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            s[t] = s[t] / (float)C;                               // mean
+            q[t] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float dl = val[t][c] - s[t];
+                q[t] += act ? dl * dl : 0.f;
+            }
+        }
+        group_sum_n<GS, NT>(q);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float rstd = 1.0f / sqrtf(q[t] / (float)C + eps);
+            float y[VEC];
+#pragma unroll
+            for (int c = 0; c < VEC; c++) y[c] = (val[t][c] - s[t]) * rstd * w[c] + bb[c];
+            if (act) *reinterpret_cast<u32x4 *>(ln_out + o[t]) = Elem<T>::pack(y);
+        }
+    };
+    auto window = [&](auto sz_tag) {
+        constexpr int SZ = decltype(sz_tag)::value;
+        constexpr int NT = SZ == 1 ? 1 : 4;
+        u32x4 raw[SZ * SZ];
+        int64_t o[SZ * SZ];
+#pragma unroll
+        for (int dy = 0; dy < SZ; dy++)
+#pragma unroll
+            for (int dx = 0; dx < SZ; dx++) {
+                o[dy * SZ + dx] = off + ((int64_t)dy * W + dx) * C;
+                raw[dy * SZ + dx] = *reinterpret_cast<const u32x4 *>(ref + o[dy * SZ + dx]);
+            }
+#pragma unroll
+        for (int i = 0; i < SZ * SZ; i += NT) finish(std::integral_constant<int, NT>{}, raw + i, o + i);
+    };
+    if (sz == 1) window(std::integral_constant<int, 1>{});
+    else if (sz == 2) window(std::integral_constant<int, 2>{});
+    else if (sz == 4) window(std::integral_constant<int, 4>{});
+    else {
+        for (int dy = 0; dy < sz; dy++)
+            for (int dx = 0; dx < sz; dx++) {
+                const int64_t o = off + ((int64_t)dy * W + dx) * C;
+                const u32x4 raw = *reinterpret_cast<const u32x4 *>(ref + o);
+                finish(std::integral_constant<int, 1>{}, &raw, &o);
+            }
+    }
+}
+
 // --------------------------------------------------------------- layernorm
 constexpr int LN_RPW = 4;   // rows per wave: their loads are issued together so that enough bytes are in flight
 
@@ -596,11 +741,17 @@ extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *split
                VTDGE_MAX_SPLITS);
     VT_REQUIRE(patches == nullptr || capacity_rows >= 0, VTDGE_ERR_ARG, "index_to_patch: negative capacity");
     hipStream_t st = (hipStream_t)stream;
+    if (patches != nullptr && (int64_t)B * Hr * Wr <= 16384) {
+        // small batches: one launch, every sample's workgroup sums the counts before it on its own
+        patch_write_kernel<true><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
+                                                    capacity_rows);
+        return check_launch("index_to_patch");
+    }
     patch_count_scan_kernel<<<1, 1024, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, offsets, lengths);
     if (int rc = check_launch("index_to_patch(count+scan)")) return rc;
     if (patches != nullptr) {
-        patch_write_kernel<<<B, 256, 0, st>>>(indices, splits, offsets, Hr, Wr, S, R, extra, patches,
-                                              capacity_rows);
+        patch_write_kernel<false><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
+                                                     capacity_rows);
         return check_launch("index_to_patch(write)");
     }
     return VTDGE_OK;
@@ -696,6 +847,43 @@ extern "C" int vtdge_decompress(const void *in, const void *sub, const int64_t *
 #undef VT_DISPATCH
 #undef VT_LAUNCH
     return check_launch("decompress");
+}
+
+extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *patches,
+                                          const int64_t *rows_dev, int64_t rows, const void *ref, void *out,
+                                          void *ln_out, const void *ln_weight, const void *ln_bias, float ln_eps,
+                                          int B, int N, int C, int W, int extra, int dtype, void *stream)
+{
+    VT_REQUIRE(in && patches && out && ref && ln_out && ln_weight && ln_bias, VTDGE_ERR_ARG,
+               "decompress_layernorm: NULL operand");
+    VT_REQUIRE(B > 0 && N > 0 && W > 0 && extra >= 0 && rows >= 0, VTDGE_ERR_ARG, "decompress_layernorm: bad sizes");
+    VT_REQUIRE((N - extra) % W == 0, VTDGE_ERR_ARG, "decompress_layernorm: N-extra=%d is not a multiple of W=%d",
+               N - extra, W);
+    if (int rc = check_channels(C, dtype, "decompress_layernorm")) return rc;
+    VT_REQUIRE(aligned16(in) && aligned16(out) && aligned16(sub) && aligned16(ref) && aligned16(ln_out) &&
+                   aligned16(ln_weight) && aligned16(ln_bias),
+               VTDGE_ERR_ARG, "decompress_layernorm: operands must be 16-byte aligned");
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(C / vec <= WAVE, VTDGE_ERR_UNSUPPORTED, "decompress_layernorm: C=%d exceeds %d (one vector per lane)",
+               C, WAVE * vec);
+    if (rows == 0) return VTDGE_OK;
+    const int gs = group_size(C / vec);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
+    hipStream_t st = (hipStream_t)stream;
+#define VT_LAUNCH(T, SUBF, GS)                                                                                      \
+    decompress_ln_kernel<T, SUBF, GS><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev,     \
+                                                              rows, (const T *)ref, (T *)out, (T *)ln_out,          \
+                                                              (const T *)ln_weight, (const T *)ln_bias, ln_eps, N,  \
+                                                              C, W, extra)
+#define VT_DISPATCH(T, GS) do { if (sub) VT_LAUNCH(T, true, GS); else VT_LAUNCH(T, false, GS); } while (0)
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_DISPATCH(T, 64); else if (gs == 32) VT_DISPATCH(T, 32); else if (gs == 16) VT_DISPATCH(T, 16); \
+         else VT_DISPATCH(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
+#undef VT_DISPATCH
+#undef VT_LAUNCH
+    return check_launch("decompress_layernorm");
 }
 
 extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,

@@ -16,6 +16,11 @@ from . import ops
 # in eager mode and inside a captured graph alike.
 _side_streams = {}
 OVERLAP = True          # module switch (benchmarks turn it off to time kernels one at a time)
+# The scatter-back of a block can also write the next block's first LayerNorm (one kernel less, 50 MB less read per
+# block).  Off by default: that LayerNorm runs on the second stream next to the routing chain and costs nothing on
+# the critical path, while the fused scatter-back is on it and slower (measured -4 % end to end at the headline
+# config); useful when `OVERLAP` is off.
+FUSE_NEXT_NORM = False
 
 
 def _side_stream(device, slot=0):
@@ -58,12 +63,14 @@ def _key_value_source(attn, x_ln, H, W, extra):
     return ops.layernorm(red, attn.norm.weight, attn.norm.bias, attn.norm.eps).view(B, -1, C)
 
 
-def block_forward(block, x, H, W, gate=None, overlap=True):
+def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=None):
     """x [B, N, C] -> [B, N, C] for a DGE transformer block (`models.dge.deit_dge.Block` or
     `models.dge.pvt_dge.Block`) in eval mode.
 
     `gate` [B, Hr, Wr, S] overrides the router's logits (used by the parity tests).
     `overlap` issues the key/value chain on a second stream next to the routing chain.
+    `x_ln` is norm1(x) when the caller already has it; `next_norm` is the LayerNorm the next block applies to this
+    block's output first: the scatter-back kernel then writes that too and the call returns (out, next_norm(out)).
     """
     dge, attn, mlp = block.dge, block.attn, block.mlp
     B, N, C = x.shape
@@ -80,7 +87,8 @@ def block_forward(block, x, H, W, gate=None, overlap=True):
     if overlap:
         side.wait_stream(main)
     with torch.cuda.stream(side):
-        x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
+        if x_ln is None:
+            x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
         kv_src = _key_value_source(attn, x_ln, H, W, extra)
         kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)                 # [B, n, 2C] = [B, n, 2, h, d]
 
@@ -107,11 +115,18 @@ def block_forward(block, x, H, W, gate=None, overlap=True):
     hid = ops.linear(q1_ln, mlp.fc1.weight, mlp.fc1.bias, act="gelu", rows_dev=rows_dev)
     q2 = ops.linear(hid, mlp.fc2.weight, mlp.fc2.bias, residual=q1, rows_dev=rows_dev)
 
-    out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
+    out_ln = None
+    if next_norm is not None and FUSE_NEXT_NORM and ops.fits_decompress_layernorm(x):
+        out, out_ln = ops.decompress_layernorm(q2, patches, x, W, extra, next_norm.weight, next_norm.bias,
+                                               next_norm.eps, sub=comp, rows_dev=rows_dev, rows=cap)
+    else:
+        out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 
     dge.states.update({"comp": comp, "input": x, "patches": patches, "batches": None, "batches_device": lengths,
                        "offsets_device": offsets, "gate": gate, "size": (H, W), "num_extra_tokens": extra,
                        "queries": q2})
+    if next_norm is not None:
+        return out, out_ln          # out_ln is None when the fused kernel does not apply: the next block normalises
     return out
 
 
@@ -135,8 +150,13 @@ def model_forward(model, images):
     x[:, 1:, :] = tok.view(B, G * G, C)
     x[:, :1, :] = model.cls_token
     x += model.pos_embed
-    for blk in model.blocks:
-        x = block_forward(blk, x, G, G)
+    x_ln = None
+    blocks = list(model.blocks)
+    for i, blk in enumerate(blocks):
+        if i + 1 < len(blocks):     # the scatter-back of this block also writes the next block's norm1
+            x, x_ln = block_forward(blk, x, G, G, x_ln=x_ln, next_norm=blocks[i + 1].norm1)
+        else:
+            x = block_forward(blk, x, G, G, x_ln=x_ln)
     cls = ops.layernorm(x[:, 0, :], model.norm.weight, model.norm.bias, model.norm.eps)
     if isinstance(model.head, torch.nn.Linear):
         return ops.linear(cls, model.head.weight, model.head.bias)
@@ -179,8 +199,13 @@ def pvt_forward(model, images):
             x += pos
         else:
             x = tok + model._get_pos_embed(pos, pe, H, W)
-        for blk in getattr(model, f"block{i + 1}"):
-            x = block_forward(blk, x, H, W)
+        x_ln = None
+        blocks = list(getattr(model, f"block{i + 1}"))
+        for bi, blk in enumerate(blocks):
+            if bi + 1 < len(blocks):
+                x, x_ln = block_forward(blk, x, H, W, x_ln=x_ln, next_norm=blocks[bi + 1].norm1)
+            else:
+                x = block_forward(blk, x, H, W, x_ln=x_ln)
         if not last:
             outputs[f"res{i + 2}"] = x.view(B, H, W, C)
         elif model.num_classes == 0:

@@ -86,6 +86,27 @@ def decompress(inp, patches, reference, width, num_extra_tokens, add_ref=True, s
     return out
 
 
+def decompress_layernorm(inp, patches, reference, width, num_extra_tokens, ln_weight, ln_bias, ln_eps=1e-6, sub=None,
+                         rows_dev=None, rows=None):
+    """Scatter (inp - sub) + reference back over the tokens, and the LayerNorm of the result: (out, LayerNorm(out))."""
+    _need_gpu(inp, patches, reference, sub, ln_weight, ln_bias)
+    inp, patches, reference = _contig(inp), _contig(patches), _contig(reference)
+    sub = None if sub is None else _contig(sub)
+    B, N, C = reference.shape
+    rows = patches.shape[0] if rows is None else rows
+    out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
+    ln_out = torch.empty_like(out)
+    call("vtdge_decompress_layernorm", ptr(inp), ptr(sub), ptr(patches), ptr(rows_dev), rows, ptr(reference), ptr(out),
+         ptr(ln_out), ptr(ln_weight), ptr(ln_bias), float(ln_eps), B, N, C, width, num_extra_tokens, dtype_code(inp),
+         stream_ptr(), tag=("decompress_ln", sub is not None, C))
+    return out, ln_out
+
+
+def fits_decompress_layernorm(x):
+    """Whether a row of x is at most 64 16-byte vectors (the fused scatter + LayerNorm holds a row in one wave)."""
+    return x.shape[-1] * x.element_size() <= 64 * 16
+
+
 def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     _need_gpu(x, weight, bias)
     x = _contig(x)
