@@ -150,6 +150,27 @@ def test_deit_tiny_fp32_model(dev, fused):
     assert rel_err(got, want) <= FP32_REL, rel_err(got, want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_model_with_fused_next_layernorm(dev, dtype):
+    """The scatter-back that also writes the next block's first LayerNorm is an option of the fused path: with it
+    the model gives the same gate choices and, the two LayerNorm kernels being one arithmetic, the same logits."""
+    from vtpack_amd import engine
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_tiny_patch16_256", dev, dtype)
+    img = synthetic_images(3, 256, seed=5, dtype=dtype).to(dev)
+    with torch.no_grad():
+        base = m(img)
+        idx = [blk.dge.states["gate"].argmax(-1).clone() for blk in m.blocks]
+        engine.FUSE_NEXT_NORM = True
+        try:
+            got = m(img)
+        finally:
+            engine.FUSE_NEXT_NORM = False
+    for blk, want in zip(m.blocks, idx):
+        assert torch.equal(blk.dge.states["gate"].argmax(-1), want)
+    assert_close(got.float(), base.float().cpu(), dtype, "logits with the fused LayerNorm")
+
+
 def test_deit_small_bf16_model(dev):
     """Config 3 at a CPU-friendly batch: DeiT-S+DGE bf16 logits within 2e-2 of the fp32 CPU path fed the same
     (bf16-rounded) weights and the same gate choices; the gate choices themselves agree with the CPU path's own
