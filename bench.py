@@ -74,7 +74,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
-            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}>"
+            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_compress":
