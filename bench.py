@@ -72,6 +72,8 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         rows, N, K = tag[4], tag[5], tag[6]
         if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
             return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}>"
+        if dt == "bf16" and K == 1536 and N % 96 == 0 and N // 96 <= 8 and rows >= 2048 and not act:
+            return f"linear_ks_kernel<{b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
@@ -337,7 +339,9 @@ def run_isolated_gemm(args, torch):
             "config": {"workload": "cfg4: 256 segments, skewed lengths in [16,256], K=384, N in {384,1152,1536}",
                        "packed_rows": L},
             "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": 2500.0, "unit": "TFLOP/s",
-                         "frac": round(ach / 2500.0, 4), "kernel": "linear_dma_kernel<unsigned short, ...>",
+                         "frac": round(ach / 2500.0, 4),
+                         "kernel": "linear_ws_kernel<24, 3, 0, true, false>" if L >= 2048
+                         else "linear_dma_kernel<unsigned short, ...>",
                          "traffic": None},
             "per_n": per_n}
 

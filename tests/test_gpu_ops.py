@@ -323,6 +323,77 @@ def test_linear_weight_stationary_matches_streaming_kernel(dev):
     assert torch.equal(ops.linear(a, w)[:2000], ops.linear(a[:2000], w))
 
 
+# The K-split weight-stationary kernel: bf16, K = 1536, N a multiple of 96, 2048 rows or more, no activation.
+@pytest.mark.parametrize("M,N", [(2048, 384), (2053, 96), (4127, 384), (9001, 768), (33000, 384), (3000, 192)])
+@pytest.mark.parametrize("epi", ["plain", "bias", "res", "bias_res"])
+def test_linear_k_split(dev, M, N, epi):
+    from vtpack_amd import ops
+    K = 1536
+    g = torch.Generator().manual_seed(3 * M + N)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.03).bfloat16()
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16()
+    res = torch.randn(M, N, generator=g).bfloat16()
+    want = a.double() @ w.double().T
+    if "bias" in epi:
+        want = want + bias.double()
+    if "res" in epi:
+        want = want + res.double()
+    got = ops.linear(a.to(dev), w.to(dev), bias.to(dev) if "bias" in epi else None,
+                     res.to(dev) if "res" in epi else None)
+    err = (got.double().cpu() - want).abs()
+    small = want.abs() < 4
+    assert float(err[small].max()) <= BF16_ABS, f"k-split linear {epi}: {float(err[small].max()):.3e}"
+    assert float((err / want.abs().clamp_min(4)).max()) <= 2 ** -7, f"k-split linear {epi} (relative)"
+
+
+@pytest.mark.parametrize("live", [0, 1, 7, 15, 16, 17, 33, 1000, 4999])
+def test_linear_k_split_device_rows(dev, live):
+    """The live row count comes from device memory: any count, down to a lone short tile, and nothing past it is
+    written."""
+    from vtpack_amd import ops
+    M, N, K = 6000, 384, 1536
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.03).bfloat16()
+    bias = torch.randn(N, generator=g).bfloat16()
+    res = torch.randn(M, N, generator=g).bfloat16()
+    rows_dev = torch.tensor([live], dtype=torch.int64, device=dev)
+    out = torch.full((M, N), 7.0, device=dev, dtype=torch.bfloat16)
+    ops.linear(a.to(dev), w.to(dev), bias.to(dev), residual=res.to(dev), rows_dev=rows_dev, out=out)
+    if live:
+        want = a[:live].double() @ w.double().T + bias.double() + res[:live].double()
+        assert abs_err(out[:live], want) <= 4 * BF16_ABS        # values up to ~10: one bf16 rounding
+    assert bool((out[live:] == 7.0).all())
+
+
+def test_linear_k_split_strided_and_repeatable(dev):
+    """Operands as column slices of wider buffers (row strides larger than the widths), and the same bytes on every
+    call: the four partial sums of a tile are added in a fixed order."""
+    from vtpack_amd import ops
+    M, N, K = 5003, 384, 1536
+    g = torch.Generator().manual_seed(23)
+    abuf = torch.randn(M, K + 64, generator=g).bfloat16().to(dev)
+    rbuf = torch.randn(M, N + 32, generator=g).bfloat16().to(dev)
+    obuf = torch.full((M, N + 8), 7.0, dtype=torch.bfloat16, device=dev)
+    w = (torch.randn(N, K, generator=g) * 0.03).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev)
+    a, res, out = abuf[:, 32:32 + K], rbuf[:, 16:16 + N], obuf[:, 4:4 + N]
+    ops.linear(a, w, bias, residual=res, out=out)
+    want = a.double() @ w.double().T + bias.double() + res.double()
+    assert abs_err(out, want) <= 4 * BF16_ABS
+    assert bool((obuf[:, :4] == 7.0).all()) and bool((obuf[:, 4 + N:] == 7.0).all())
+    first = out.clone()
+    for _ in range(3):
+        ops.linear(a, w, bias, residual=res, out=out)
+        assert torch.equal(out, first)
+    # fewer than 2048 rows go to the streaming kernel: the same sum in another order, so a last bit may differ
+    few = torch.empty((2000, N), dtype=torch.bfloat16, device=dev)
+    ops.linear(a[:2000], w, bias, residual=res[:2000], out=few)
+    diff = (first[:2000].float() - few.float()).abs()
+    assert float((diff / few.float().abs().clamp_min(2.0 ** -6)).max()) <= 2.0 ** -6
+
+
 # ------------------------------------------------------------------ attention / sparse gemm
 def _lengths(seed, B, lo, hi):
     return rng(seed).randint(lo, hi + 1, size=B).astype(np.int64)

@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <utility>
 
 #include "../../include/vtdge.h"
 
@@ -127,9 +128,73 @@ template <int N> __device__ __forceinline__ void wait_vmcnt()
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+// one direct load: 64 lanes x 16 B from base + the per-lane byte offset to LDS bytes [lds_addr, lds_addr + 1024)
+__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base)
+                 : "memory", "m0");
+}
+// the same with a compile-time byte offset (0 .. 4095) added to the global address.  The instruction adds its
+// immediate to the LDS address too, so that is lowered by as much first: lds_addr must be at least IMM.
+template <int IMM> __device__ __forceinline__ void dma16_imm(const void *base, uint32_t off, uint32_t lds_addr)
+{
+    static_assert(IMM >= 0 && IMM < 4096, "immediate offset of a global load");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3" ::"s"(lds_addr - IMM),
+                 "v"(off), "s"(base), "n"(IMM)
+                 : "memory", "m0");
+}
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N-1>{}): a loop whose index is a constant expression
+template <class F, int... I> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F> __device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+// makes a lane constant opaque at this point, so address arithmetic built on it is redone where it is used instead
+// of being kept in registers for the whole kernel
+__device__ __forceinline__ int fresh(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform runtime n, rounded down to a multiple of 6 and to at most 42 (waiting for
+// fewer operations in flight than allowed is always safe).  A balanced tree of three compares: the immediate of
+// s_waitcnt cannot come from a register.
+__device__ __forceinline__ void wait_vmcnt_dyn(int n)
+{
+    if (n >= 24) {
+        if (n >= 36) {
+            if (n >= 42) wait_vmcnt<42>();
+            else wait_vmcnt<36>();
+        } else {
+            if (n >= 30) wait_vmcnt<30>();
+            else wait_vmcnt<24>();
+        }
+    } else {
+        if (n >= 12) {
+            if (n >= 18) wait_vmcnt<18>();
+            else wait_vmcnt<12>();
+        } else {
+            if (n >= 6) wait_vmcnt<6>();
+            else wait_vmcnt<0>();
+        }
+    }
+}
+
 __device__ __forceinline__ void block_barrier()
 {
     asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+// barrier that also publishes this wave's LDS accesses (all of them complete first) but, unlike __syncthreads(),
+// leaves vector-memory operations - the prefetches - in flight
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }

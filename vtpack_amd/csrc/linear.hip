@@ -199,6 +199,12 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
 int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
                      void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act, hipStream_t st);
 
+// K-split weight-stationary variant for bf16, K = 1536, narrow N (linear_ks.hip)
+bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
+                          const void *bias, const void *res, const void *out);
+int launch_linear_ks(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
+                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st);
+
 }  // namespace vtdge
 
 using namespace vtdge;
@@ -222,6 +228,8 @@ extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const voi
     hipStream_t st = (hipStream_t)stream;
     if (linear_ws_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
         return launch_linear_ws(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
+    if (linear_ks_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
+        return launch_linear_ks(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, st);
     if (linear_dma_applicable(lda, ldr, ldo, N, K, esz, bias, residual, out)) {
         if (dtype == VTDGE_F32)
             return launch_linear_dma<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);

@@ -45,20 +45,6 @@ __device__ long long ws_dbg[4][64];
 #define VT_WS_STAMP(i) do { } while (0)
 #endif
 
-// one direct load: 64 lanes x 16 B from base + the per-lane byte offset to LDS bytes [lds_addr, lds_addr + 1024)
-__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds_addr)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base)
-                 : "memory", "m0");
-}
-// makes a lane constant opaque at this point, so address arithmetic built on it is redone where it is used instead
-// of being kept in registers for the whole kernel
-__device__ __forceinline__ int fresh(int v)
-{
-    asm volatile("" : "+v"(v));
-    return v;
-}
-
 // D = W_frag * A_frag^T (+ D).  The stationary fragment sits in accumulation registers (A) or vector registers (V);
 // Z starts a new sum.  Issued from assembly so the register classes are exactly these.
 __device__ __forceinline__ void mma_a(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
@@ -78,30 +64,6 @@ __device__ __forceinline__ void mma_v_fresh(f32x16 &d, const u32x4 &wfrag, const
 __device__ __forceinline__ void mma_az(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
 {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "a"(wfrag), "v"(afrag));
-}
-
-// s_waitcnt vmcnt(n) for a wave-uniform runtime n, rounded down to a multiple of 6 and to at most 42 (waiting for
-// fewer operations in flight than allowed is always safe).  A balanced tree of three compares: the immediate of
-// s_waitcnt cannot come from a register.
-__device__ __forceinline__ void wait_vmcnt_dyn(int n)
-{
-    if (n >= 24) {
-        if (n >= 36) {
-            if (n >= 42) wait_vmcnt<42>();
-            else wait_vmcnt<36>();
-        } else {
-            if (n >= 30) wait_vmcnt<30>();
-            else wait_vmcnt<24>();
-        }
-    } else {
-        if (n >= 12) {
-            if (n >= 18) wait_vmcnt<18>();
-            else wait_vmcnt<12>();
-        } else {
-            if (n >= 6) wait_vmcnt<6>();
-            else wait_vmcnt<0>();
-        }
-    }
 }
 
 // State of one epilogue unit: two output elements of a lane on their way from the accumulator to bf16.
@@ -308,14 +270,14 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         VT_WS_STAMP(40);
         wait_vmcnt<2 * NL>();                  // round 0 has landed
         VT_WS_STAMP(41);
-        __syncthreads();
+        lds_barrier();
         // the bias values are consumed here as far as the compiler is concerned: their loads are issued above and
         // waited for now, not next to their first real use in the middle of the pipeline
 #pragma unroll
         for (int j = 0; j < NB; j++) asm volatile("" : "+v"(wb[j]));
         read_w(0, w);
         VT_WS_STAMP(42);
-        __syncthreads();                       // slots 0..3 are free
+        lds_barrier();                       // slots 0..3 are free
         issue_w(2, 1, 0);
         issue_w(3, 1, 1);
         issue_w(0, 2, 2);
@@ -323,10 +285,10 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         VT_WS_STAMP(43);
         wait_vmcnt<2 * NL>();                  // round 1 has landed
         VT_WS_STAMP(44);
-        __syncthreads();
+        lds_barrier();
         read_w(1, w < 2 ? 4 + w : w - 2);
         VT_WS_STAMP(45);
-        __syncthreads();                       // slots 4, 5, 0, 1 are free
+        lds_barrier();                       // slots 4, 5, 0, 1 are free
         issue_w(2, 2, 4);
         issue_w(3, 2, 5);
 #pragma unroll
@@ -335,10 +297,10 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         VT_WS_STAMP(46);
         wait_vmcnt_dyn(issued);                // round 2 has landed (all but the tiles of A)
         VT_WS_STAMP(47);
-        __syncthreads();
+        lds_barrier();
         read_w(2, 2 + w);
         VT_WS_STAMP(48);
-        __syncthreads();                       // slots 2..5 are free
+        lds_barrier();                       // slots 2..5 are free
     }
     VT_WS_STAMP(1);
     // ---- rest of the prologue: first residual tiles, remaining first tiles of A
