@@ -93,7 +93,9 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return "sparse_attention_bf16_d64_resident_kernel" if tag[4] <= 288 else "sparse_attention_bf16_d64_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
-        return f"router_kernel<{T}, 4, {gs(tag[1])}>"     # region size 4 in every model of these workloads
+        return f"router_kernel<{T}, 4, {gs(tag[1])}, false>"     # region size 4 in every model of these workloads
+    if name == "vtdge_router_layernorm":
+        return f"router_kernel<{T}, 4, {gs(tag[1])}, true>"
     if name == "vtdge_index_to_patch":
         return "patch_write_kernel<true>"      # one launch for batch * regions <= 16384 (all workloads here)
     return name
@@ -137,6 +139,8 @@ def algorithmic_work(name, tag, esz, geo):
         return "hbm", 2.0 * rows * tag[3] * esz
     if name == "vtdge_router":
         return "hbm", B * (N - geo["extra"]) * C * esz
+    if name == "vtdge_router_layernorm":
+        return "hbm", 2.0 * B * N * C * esz              # every token read once, its LayerNorm written once
     if name == "vtdge_index_to_patch":
         return "hbm", 8.0 * B * geo["regions"] + 32 * L + 8 * B
     return "hbm", 0.0

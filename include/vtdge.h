@@ -58,6 +58,16 @@ const char *vtdge_last_error(void);
 int vtdge_router(const void *x, const void *weight, const void *bias, void *gate, int64_t *indices,
                  int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream);
 
+/* The router and the block's first LayerNorm in one pass over x: gate / indices as vtdge_router, plus
+ *   ln_out [B, extra + H*W, C] = LayerNorm(x) * ln_weight + ln_bias   (every token, the extra ones included).
+ * Replaces DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75) together with norm1 applied to
+ * all tokens (vtpack/models/dge/deit_dge.py:127); both results are bit-identical to vtdge_router and
+ * vtdge_layernorm.  R must be 4 or 2 and a row must fit one 16-byte vector per lane (C <= 512 in bf16, 256 in
+ * fp32); VTDGE_ERR_UNSUPPORTED otherwise. */
+int vtdge_router_layernorm(const void *x, const void *weight, const void *bias, void *gate, int64_t *indices,
+                           const void *ln_weight, const void *ln_bias, float ln_eps, void *ln_out, int B, int H,
+                           int W, int C, int extra, int R, int S, int dtype, void *stream);
+
 /* Gate indices -> packed query descriptors.
  * Replaces grained_sample_index_to_patch
  * (vtpack/layers/csrc/grained_sample/grained_sample.cu:302-345, kernel :146-196).

@@ -171,6 +171,27 @@ def test_model_with_fused_next_layernorm(dev, dtype):
     assert_close(got.float(), base.float().cpu(), dtype, "logits with the fused LayerNorm")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_model_router_with_layernorm_is_the_same_model(dev, dtype):
+    """The router that also writes the first LayerNorm (an option of the fused path) and the two separate kernels
+    are the same arithmetic: identical logits and gate choices."""
+    from vtpack_amd import engine
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_tiny_patch16_256", dev, dtype)
+    img = synthetic_images(3, 256, seed=6, dtype=dtype).to(dev)
+    with torch.no_grad():
+        apart = m(img)
+        idx = [blk.dge.states["gate"].argmax(-1).clone() for blk in m.blocks]
+        engine.FUSE_ROUTER_NORM = True
+        try:
+            fused = m(img)
+        finally:
+            engine.FUSE_ROUTER_NORM = False
+    for blk, want in zip(m.blocks, idx):
+        assert torch.equal(blk.dge.states["gate"].argmax(-1), want)
+    assert torch.equal(fused, apart)
+
+
 def test_deit_small_bf16_model(dev):
     """Config 3 at a CPU-friendly batch: DeiT-S+DGE bf16 logits within 2e-2 of the fp32 CPU path fed the same
     (bf16-rounded) weights and the same gate choices; the gate choices themselves agree with the CPU path's own

@@ -205,6 +205,46 @@ def test_router_gate_and_indices(dev, dtype, B, H, W, extra, C):
     assert torch.equal(indices.cpu(), gate.float().cpu().argmax(-1))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,W,extra,C,R", [(8, 16, 16, 1, 192, 4), (3, 8, 12, 0, 64, 4), (5, 16, 16, 2, 384, 4),
+                                             (2, 32, 32, 1, 384, 4), (4, 8, 8, 1, 128, 2), (2, 4, 4, 1, 512, 4),
+                                             (3, 4, 8, 0, 256, 2)])
+def test_router_with_layernorm(dev, dtype, B, H, W, extra, C, R):
+    """One pass over x gives the router's outputs and LayerNorm of every token: bit for bit what the two separate
+    kernels give, and the LayerNorm within tolerance of the library routine."""
+    from vtpack_amd import ops
+    if dtype == torch.float32 and C > 256:
+        pytest.skip("one 16-byte vector per lane and row: at most 256 fp32 channels")
+    x = randn(121, B, extra + H * W, C) * 1.5 + 0.3
+    w, b = randn(122, 3, C) * 0.3, randn(123, 3) * 0.1
+    lw, lb = randn(124, C) * 0.2 + 1, randn(125, C) * 0.1
+    if dtype == torch.bfloat16:
+        x, w, b, lw, lb = (bf16_round(t) for t in (x, w, b, lw, lb))
+    xd, wd, bd, lwd, lbd = (_t(t, dev, dtype) for t in (x, w, b, lw, lb))
+    assert ops.fits_router_layernorm(xd, R)
+    gate, indices, x_ln = ops.router_layernorm(xd, wd, bd, H, W, R, lwd, lbd, 1e-6)
+    gate0, indices0 = ops.router(xd, wd, bd, H, W, R)
+    assert torch.equal(gate, gate0) and torch.equal(indices, indices0)
+    assert torch.equal(x_ln, ops.layernorm(xd, lwd, lbd, 1e-6))
+    want = torch.nn.functional.layer_norm(torch.from_numpy(x), (C,), torch.from_numpy(lw), torch.from_numpy(lb), 1e-6)
+    assert_close(x_ln.float(), want, dtype, "router + layernorm")
+
+
+def test_router_with_layernorm_refuses_what_it_cannot_do(dev):
+    from vtpack_amd import ops
+    from vtpack_amd._lib import VtdgeError
+    x = torch.zeros(2, 1 + 64, 768, device=dev, dtype=torch.bfloat16)
+    w, b = torch.zeros(3, 768, device=dev, dtype=torch.bfloat16), torch.zeros(3, device=dev, dtype=torch.bfloat16)
+    lw = torch.ones(768, device=dev, dtype=torch.bfloat16)
+    assert not ops.fits_router_layernorm(x, 4)
+    with pytest.raises(VtdgeError):
+        ops.router_layernorm(x, w, b, 8, 8, 4, lw, lw, 1e-6)
+    x = torch.zeros(2, 1 + 64, 384, device=dev, dtype=torch.bfloat16)
+    assert not ops.fits_router_layernorm(x, 8)
+    with pytest.raises(VtdgeError):
+        ops.router_layernorm(x, w[:, :384].contiguous(), b, 8, 8, 8, lw[:384].contiguous(), lw[:384].contiguous(), 1e-6)
+
+
 # ------------------------------------------------------------------ layernorm / linear
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,C", [(1, 192), (257, 384), (1000, 768), (33, 64)])

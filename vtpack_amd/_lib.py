@@ -25,6 +25,7 @@ _f = ctypes.c_float
 # name -> argtypes, in the order of include/vtdge.h
 SIGNATURES = {
     "vtdge_router": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "vtdge_router_layernorm": [_p, _p, _p, _p, _p, _p, _p, _f, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_index_to_patch": [_p, _p, _i, _i, _i, _i, _i, _i, _p, _l, _p, _p, _p],
     "vtdge_index_to_patch_dense": [_p, _i, _i, _i, _i, _i, _i, _p, _p],
     "vtdge_compress": [_p, _p, _p, _l, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p],

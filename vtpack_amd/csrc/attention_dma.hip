@@ -10,6 +10,7 @@
 //   * the softmax works in the log2 domain: p = exp2(fma(s, scale*log2(e), -m)); the running maximum is taken on
 //     the raw scores (scale > 0), and key masking is only applied in a stage that contains the end of the keys.
 #include "common.h"
+#include <stdlib.h>
 
 namespace vtdge {
 
@@ -226,11 +227,11 @@ __device__ __forceinline__ void attn_stage_resident_nb(int nb, const unsigned ch
 __global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_resident_kernel(
     const bf16_t *__restrict__ q, int64_t q_rs, int64_t q_hs, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, int64_t kv_bs, int64_t kv_ts, int64_t kv_hs, const int64_t *__restrict__ offsets,
-    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale)
+    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale, int B, int h, int order)
 {
     constexpr int MAXV = 9;          // 16-byte V chunks per thread: covers n_pad = 288
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int b = blockIdx.x, head = blockIdx.y;
+    const int b = order ? blockIdx.x / h : blockIdx.x % B, head = order ? blockIdx.x % h : blockIdx.x / B;
     const int64_t row0 = offsets[b];
     const int Lb = (int)(offsets[b + 1] - row0);
     if (Lb <= 0) return;
@@ -463,9 +464,15 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
             }
             attr_r = true;
         }
-        dim3 grid_r((unsigned)B, (unsigned)h), block_r(256);
+        static int order = -1;
+        if (order < 0) {
+            const char *e = getenv("VTDGE_ATT_ORDER");
+            order = e ? atoi(e) : 0;
+        }
+        dim3 grid_r((unsigned)(B * h)), block_r(256);
         kern_r<<<grid_r, block_r, lds_r, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v,
-                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale);
+                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale, B, h,
+                                               order);
         return check_launch("sparse_attention");
     }
     const size_t lds = 2 * (size_t)ABUF;

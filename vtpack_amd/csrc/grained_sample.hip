@@ -40,14 +40,70 @@ template <int GS> __device__ __forceinline__ float group_sum(float v)
     }
 }
 
+// LayerNorm of NR rows at once, one 16-byte vector of each row per lane of a GS-lane group (`active` false: the
+// lane holds no channels and only takes part in the sums).  dst(t) is where the lane's vector of row t goes.
+template <typename T, int GS, int NR, class F>
+__device__ __forceinline__ void layernorm_rows(const u32x4 (&raw)[NR], bool active, const T *__restrict__ w,
+                                               const T *__restrict__ bsrc, float eps, int C, F &&dst)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    float s[NR];
+#pragma unroll
+    for (int t = 0; t < NR; t++) {
+        float f[VEC];
+        Elem<T>::unpack(raw[t], f);
+        s[t] = 0.f;
+#pragma unroll
+        for (int c = 0; c < VEC; c++) s[t] += f[c];
+    }
+    group_sum_n<GS, NR>(s);
+    float q[NR];
+#pragma unroll
+    for (int t = 0; t < NR; t++) {
+        s[t] = s[t] / (float)C;      // mean
+        float f[VEC];
+        Elem<T>::unpack(raw[t], f);
+        q[t] = 0.f;
+        if (active) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float dlt = f[c] - s[t];
+                q[t] += dlt * dlt;
+            }
+        }
+    }
+    group_sum_n<GS, NR>(q);
+    if (!active) return;          // after the last reduction
+    float ww[VEC], bb[VEC];
+    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(w), ww);
+    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(bsrc), bb);
+#pragma unroll
+    for (int t = 0; t < NR; t++) {
+        const float rstd = 1.0f / sqrtf(q[t] / (float)C + eps);
+        float f[VEC], y[VEC];
+        Elem<T>::unpack(raw[t], f);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) y[c] = (f[c] - s[t]) * rstd * ww[c] + bb[c];
+        *reinterpret_cast<u32x4 *>(dst(t)) = Elem<T>::pack(y);
+    }
+}
+
 // ------------------------------------------------------------------ router
 // One wave per region.  Replaces AvgPool2d(R,R) -> Linear(C,S) -> argmax
 // (vtpack/layers/dge.py:145-150, :75).
-template <typename T, int RS, int GS>   // RS = region size known at compile time (all window loads in flight), 0 = generic
+//
+// LNF: the wave also writes LayerNorm(x) of the tokens it has just read (and the wave of a sample's first region
+// that of the sample's extra tokens): the block's first LayerNorm (vtpack/models/dge/deit_dge.py:127) without a
+// second pass over x.  Same arithmetic as layernorm_kernel (two-pass statistics in fp32, the same reduction
+// tree).  Needs RS > 0 and a row that fits one 16-byte vector per lane of the group.
+template <typename T, int RS, int GS, bool LNF = false>   // RS = region size known at compile time (all window loads in flight), 0 = generic
 __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, const T *__restrict__ weight,
                                                       const T *__restrict__ bias, T *__restrict__ gate,
                                                       int64_t *__restrict__ indices, int B, int H, int W,
-                                                      int C, int extra, int R, int S)
+                                                      int C, int extra, int R, int S,
+                                                      const T *__restrict__ ln_w = nullptr,
+                                                      const T *__restrict__ ln_b = nullptr, float eps = 0.f,
+                                                      T *__restrict__ ln_out = nullptr)
 {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & (GS - 1);
@@ -66,6 +122,55 @@ __global__ __launch_bounds__(256) void router_kernel(const T *__restrict__ x, co
 #pragma unroll
     for (int s = 0; s < VTDGE_MAX_SPLITS; s++) part[s] = 0.f;
 
+    if constexpr (LNF) {
+        // one vector per lane (the host launches this variant only when nvec <= GS); every lane of the group takes
+        // part in the reductions, lanes past the row with zeros
+        static_assert(RS > 0, "the fused LayerNorm needs the region size at compile time");
+        const bool act = lane < nvec;
+        const int v = act ? lane : 0;
+        const int64_t tok0 = (int64_t)(ry * R) * W + rx * R + extra;
+        const T *base = xb + tok0 * C + v * VEC;
+        u32x4 raw[RS * RS];
+#pragma unroll
+        for (int t = 0; t < RS * RS; t++) {
+            raw[t] = u32x4{0u, 0u, 0u, 0u};
+            if (act) raw[t] = *reinterpret_cast<const u32x4 *>(base + ((int64_t)(t / RS) * W + (t % RS)) * C);
+        }
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+#pragma unroll
+        for (int t = 0; t < RS * RS; t++) {
+            float f[VEC];
+            Elem<T>::unpack(raw[t], f);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) acc[i] += f[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = Elem<T>::round(acc[i] / area);
+        if (act) {
+#pragma unroll
+            for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
+                if (s < S) {
+                    float w[VEC];
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(weight + (int64_t)s * C + v * VEC), w);
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) part[s] += acc[i] * w[i];
+                }
+            }
+        }
+        T *ob = ln_out + (int64_t)b * N * C + tok0 * C + v * VEC;
+        layernorm_rows<T, GS, RS * RS>(raw, act, ln_w + v * VEC, ln_b + v * VEC, eps, C,
+                                       [&](int t) { return ob + ((int64_t)(t / RS) * W + (t % RS)) * C; });
+        if (rr == 0) {           // the sample's extra tokens (a branch the whole group takes or not)
+            for (int e = 0; e < extra; e++) {
+                u32x4 one[1] = {u32x4{0u, 0u, 0u, 0u}};
+                if (act) one[0] = *reinterpret_cast<const u32x4 *>(xb + (int64_t)e * C + v * VEC);
+                T *oe = ln_out + (int64_t)b * N * C + (int64_t)e * C + v * VEC;
+                layernorm_rows<T, GS, 1>(one, act, ln_w + v * VEC, ln_b + v * VEC, eps, C, [&](int) { return oe; });
+            }
+        }
+    } else
     for (int v = lane; v < nvec; v += GS) {
         float acc[VEC];
 #pragma unroll
@@ -179,12 +284,15 @@ __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *_
 }
 
 // Step 2: one workgroup per sample.  The per-region query counts go through an
-// LDS-staged wavefront prefix sum (256 regions per pass); each thread then
-// emits the descriptors of its own region at offsets[b] + extra + prefix.
+// LDS-staged wavefront prefix sum (256 regions per pass); then every thread emits
+// one descriptor per turn (row j of the sample: its region by binary search in the
+// prefix sums), so a workgroup writes 256 consecutive 32-byte rows at a time.
 //
 // FUSED: the workgroup also finds its own first row, as the sum of the query counts of all samples before it (it
 // reads their gate indices itself: a few KB out of L2 for the batch sizes this variant is launched for), and writes
 // offsets / lengths; no first step then, and no dependency between workgroups.
+typedef long long i64x2 __attribute__((ext_vector_type(2)));
+
 template <bool FUSED>
 __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restrict__ indices,
                                                            const int64_t *__restrict__ splits,
@@ -196,6 +304,7 @@ __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restr
     __shared__ int carry_s;
     __shared__ int split_s[VTDGE_MAX_SPLITS];
     __shared__ int64_t before_s[4];
+    __shared__ int start_s[256], ps_s[256];
     const int b = blockIdx.x;
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int nreg = Hr * Wr;
@@ -244,26 +353,37 @@ __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restr
         }
         if (lane == 63) wave_tot[wid] = inc;
         __syncthreads();
-        int before = carry_s;
+        const int first = carry_s;                 // rows of the regions of earlier passes
+        int before = first;
         for (int w = 0; w < wid; w++) before += wave_tot[w];
-        if (r < nreg) {
-            const int ry = r / Wr, rx = r % Wr;
-            const int step = R / ps;
-            int64_t row = row0 + extra + before + inc - cnt;
-            for (int dy = 0; dy < ps; dy++) {
-                for (int dx = 0; dx < ps; dx++, row++) {
-                    if (row < capacity) {
-                        int64_t *p = patches + 4 * row;
-                        p[0] = b;
-                        p[1] = (int64_t)ry * R + dy * step;
-                        p[2] = (int64_t)rx * R + dx * step;
-                        p[3] = step;
-                    }
-                }
+        // first row of the region (or, past the last region, one past the last row of the pass) and its split
+        start_s[threadIdx.x] = before + inc - cnt;
+        ps_s[threadIdx.x] = ps;
+        __syncthreads();
+        const int nr = min(256, nreg - base);
+        const int last = start_s[nr - 1] + ps_s[nr - 1] * ps_s[nr - 1];
+        // one descriptor per thread and turn: the region of row j is the last one that starts at or before j
+        for (int j = first + threadIdx.x; j < last; j += 256) {
+            int lo = 0, hi = nr - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (start_s[mid] <= j) lo = mid;
+                else hi = mid - 1;
+            }
+            const int rps = ps_s[lo], local = j - start_s[lo];
+            const int rg = base + lo, ry = rg / Wr, rx = rg % Wr;
+            const int step = R / rps, dy = local / rps, dx = local - dy * rps;
+            const int64_t row = row0 + extra + j;
+            if (row < capacity) {
+                i64x2 *p = reinterpret_cast<i64x2 *>(patches + 4 * row);
+                const i64x2 lo2 = {(int64_t)b, (int64_t)ry * R + dy * step};
+                const i64x2 hi2 = {(int64_t)rx * R + dx * step, (int64_t)step};
+                p[0] = lo2;
+                p[1] = hi2;
             }
         }
         __syncthreads();
-        if (threadIdx.x == 255) carry_s = before + inc;
+        if (threadIdx.x == 0) carry_s = last;
         __syncthreads();
     }
     if constexpr (FUSED) {
@@ -731,6 +851,45 @@ extern "C" int vtdge_router(const void *x, const void *weight, const void *bias,
     return check_launch("router");
 }
 
+extern "C" int vtdge_router_layernorm(const void *x, const void *weight, const void *bias, void *gate,
+                                      int64_t *indices, const void *ln_weight, const void *ln_bias, float ln_eps,
+                                      void *ln_out, int B, int H, int W, int C, int extra, int R, int S, int dtype,
+                                      void *stream)
+{
+    VT_REQUIRE(x && weight && bias && indices && ln_weight && ln_bias && ln_out, VTDGE_ERR_ARG,
+               "router_layernorm: NULL operand");
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && extra >= 0, VTDGE_ERR_ARG, "router_layernorm: bad sizes");
+    VT_REQUIRE(R == 4 || R == 2, VTDGE_ERR_UNSUPPORTED, "router_layernorm: region size %d (4 or 2 only)", R);
+    VT_REQUIRE(H % R == 0 && W % R == 0, VTDGE_ERR_ARG, "router_layernorm: H=%d, W=%d not multiples of region %d", H,
+               W, R);
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "router_layernorm: S=%d outside [1,%d]", S,
+               VTDGE_MAX_SPLITS);
+    if (int rc = check_channels(C, dtype, "router_layernorm")) return rc;
+    const int nvec = C / (dtype == VTDGE_BF16 ? 8 : 4);
+    VT_REQUIRE(nvec <= 64, VTDGE_ERR_UNSUPPORTED, "router_layernorm: C=%d exceeds one 16-byte vector per lane", C);
+    VT_REQUIRE(aligned16(x) && aligned16(weight) && aligned16(ln_weight) && aligned16(ln_bias) && aligned16(ln_out),
+               VTDGE_ERR_ARG, "router_layernorm: operands must be 16-byte aligned");
+    const int64_t regions = (int64_t)B * (H / R) * (W / R);
+    const int gs = group_size(nvec);
+    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
+    hipStream_t st = (hipStream_t)stream;
+#define VT_LAUNCH(T, RS, GS)                                                                                  \
+    router_kernel<T, RS, GS, true><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias,  \
+                                                           (T *)gate, indices, B, H, W, C, extra, R, S,       \
+                                                           (const T *)ln_weight, (const T *)ln_bias, ln_eps,  \
+                                                           (T *)ln_out)
+#define VT_REGION(T, GS) \
+    do { if (R == 4) VT_LAUNCH(T, 4, GS); else VT_LAUNCH(T, 2, GS); } while (0)
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_REGION(T, 64); else if (gs == 32) VT_REGION(T, 32); else if (gs == 16) VT_REGION(T, 16); \
+         else VT_REGION(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
+#undef VT_REGION
+#undef VT_LAUNCH
+    return check_launch("router_layernorm");
+}
+
 extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *splits, int B, int Hr, int Wr, int S,
                                     int R, int extra, int64_t *patches, int64_t capacity_rows, int64_t *offsets,
                                     int64_t *lengths, void *stream)
@@ -740,6 +899,8 @@ extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *split
     VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "index_to_patch: S=%d outside [1,%d]", S,
                VTDGE_MAX_SPLITS);
     VT_REQUIRE(patches == nullptr || capacity_rows >= 0, VTDGE_ERR_ARG, "index_to_patch: negative capacity");
+    VT_REQUIRE((reinterpret_cast<uintptr_t>(patches) & 15u) == 0, VTDGE_ERR_ARG,
+               "index_to_patch: patches must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     if (patches != nullptr && (int64_t)B * Hr * Wr <= 16384) {
         // small batches: one launch, every sample's workgroup sums the counts before it on its own

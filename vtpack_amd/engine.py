@@ -21,6 +21,11 @@ OVERLAP = True          # module switch (benchmarks turn it off to time kernels 
 # the critical path, while the fused scatter-back is on it and slower (measured -4 % end to end at the headline
 # config); useful when `OVERLAP` is off.
 FUSE_NEXT_NORM = False
+# The router reads every spatial token anyway and can write the block's first LayerNorm of all tokens on the way
+# (one pass over x less, one kernel less).  Off by default as well: one wave then loads, normalises and stores a
+# whole region with nothing to overlap the three phases (30 us against 22 us for the two kernels side by side at the
+# headline config), and both chains of the block wait for it.
+FUSE_ROUTER_NORM = False
 
 
 def _side_stream(device, slot=0):
@@ -83,6 +88,11 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
     main = torch.cuda.current_stream(x.device)
     side = _side_stream(x.device, main.cuda_stream) if overlap else main
 
+    fuse_rn = FUSE_ROUTER_NORM and gate is None and x_ln is None and ops.fits_router_layernorm(x, R)
+    if fuse_rn:
+        gate, indices, x_ln = ops.router_layernorm(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R,
+                                                   n1.weight, n1.bias, n1.eps)
+
     # key/value chain (second stream)
     if overlap:
         side.wait_stream(main)
@@ -93,10 +103,11 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
         kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)                 # [B, n, 2C] = [B, n, 2, h, d]
 
     # routing chain (caller's stream)
-    if gate is None:
-        gate, indices = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
-    else:
-        indices = gate.argmax(dim=-1)
+    if not fuse_rn:
+        if gate is None:
+            gate, indices = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
+        else:
+            indices = gate.argmax(dim=-1)
     cap = B * N
     patches, offsets, lengths = ops.index_to_patch(indices, dge.splits, R, extra, capacity=cap)
     rows_dev = offsets[B:]

@@ -40,6 +40,31 @@ def router(x, weight, bias, H, W, region_size, want_gate=True):
     return gate, indices
 
 
+def fits_router_layernorm(x, region_size):
+    """Whether the router can also write LayerNorm(x): region size 4 or 2, one 16-byte vector per lane and row."""
+    return region_size in (2, 4) and x.shape[-1] * x.element_size() <= 64 * 16
+
+
+def router_layernorm(x, weight, bias, H, W, region_size, ln_weight, ln_bias, ln_eps, want_gate=True):
+    """`router` and LayerNorm of every token of x in one pass: (gate or None, indices, LayerNorm(x)).
+
+    vtpack/layers/dge.py:145-150, :75 and norm1 of vtpack/models/dge/deit_dge.py:127."""
+    _need_gpu(x, weight, bias, ln_weight, ln_bias)
+    x, weight, bias = _contig(x), _contig(weight), _contig(bias)
+    B, N, C = x.shape
+    S = weight.shape[0]
+    extra = N - H * W
+    Hr, Wr = H // region_size, W // region_size
+    gate = torch.empty((B, Hr, Wr, S), dtype=x.dtype, device=x.device) if want_gate else None
+    indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
+    ln_out = torch.empty_like(x)
+    weight, bias = weight.to(x.dtype), bias.to(x.dtype)
+    call("vtdge_router_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(gate), ptr(indices),
+         ptr(_contig(ln_weight).to(x.dtype)), ptr(_contig(ln_bias).to(x.dtype)), float(ln_eps), ptr(ln_out), B, H, W,
+         C, extra, region_size, S, dtype_code(x), stream_ptr(), tag=("router_layernorm", C, B * N))
+    return gate, indices, ln_out
+
+
 def index_to_patch(indices, splits, region_size, num_extra_tokens, capacity=None):
     """Device-only compaction: (patches [capacity,4], offsets [B+1], lengths [B]), all on the GPU."""
     _need_gpu(indices, splits)
