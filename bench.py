@@ -67,7 +67,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
     T = "unsigned short" if dt == "bf16" else "float"
     esz = 2 if dt == "bf16" else 4
     b = lambda v: "true" if v else "false"  # noqa: E731
-    if name == "vtdge_linear":
+    if name in ("vtdge_linear", "vtdge_linear_prepacked"):
         act = 1 if tag[1] == "gelu" else 0
         rows, N, K = tag[4], tag[5], tag[6]
         if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
@@ -120,7 +120,7 @@ def algorithmic_work(name, tag, esz, geo):
 
     geo: dict with B, N, C, L (live packed rows), regions and extra of the block the launch belongs to."""
     B, N, C, L = geo["B"], geo["N"], geo["C"], geo["L"]
-    if name == "vtdge_linear":
+    if name in ("vtdge_linear", "vtdge_linear_prepacked"):
         _, _, _, _, rows, Nn, K, packed = tag
         M = L if packed else rows
         return "mfma", 2.0 * M * Nn * K

@@ -142,6 +142,23 @@ int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, co
                  int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K,
                  int act, int dtype, void *stream);
 
+/* The same Linear with a packed copy of W beside it.  The weight-stationary kernels keep a strip of W in registers
+ * for the life of a workgroup; from a copy laid out in the order of those registers they fill them with contiguous
+ * loads (half the start-up time of a launch).  The weights of an nn.Linear (vtpack/models/dge/deit_dge.py:70-74,
+ * :38-44) do not change between calls at inference, so a caller packs them once:
+ *   vtdge_linear_packed_size  *bytes = size of the packed copy of W [N, K], or 0 when no kernel for this shape uses
+ *                             one (pass packed = NULL then)
+ *   vtdge_linear_prepack      fills `packed` (16-byte aligned, *bytes long) from W; VTDGE_ERR_UNSUPPORTED when the
+ *                             size is 0
+ *   vtdge_linear_prepacked    vtdge_linear with `packed` (nullable; must have been made from this W).  W itself is
+ *                             still required: the kernels chosen for few rows read it.
+ * Results are bit-identical with and without the packed copy. */
+int vtdge_linear_packed_size(int N, int K, int dtype, int64_t *bytes);
+int vtdge_linear_prepack(const void *W, int N, int K, int dtype, void *packed, void *stream);
+int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,
+                           const void *residual, int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev,
+                           int64_t rows, int N, int K, int act, int dtype, void *stream);
+
 /* Sparse attention of packed queries against each sample's full K/V:
  *   out[rows of sample i, head a] = softmax(scale * Q_i,a K_i,a^T) V_i,a
  * Replaces batched_sparse_attention_forward

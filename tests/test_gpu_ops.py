@@ -434,6 +434,53 @@ def test_linear_k_split_strided_and_repeatable(dev):
     assert float((diff / few.float().abs().clamp_min(2.0 ** -6)).max()) <= 2.0 ** -6
 
 
+@pytest.mark.parametrize("M,N,K,epi", [(4127, 384, 384, "bias"), (9000, 1152, 384, "bias_gelu"), (2049, 768, 384, "bias_res"),
+                                       (33000, 1536, 384, "plain"), (4127, 384, 1536, "bias_res"), (2053, 96, 1536, "bias"),
+                                       (9001, 768, 1536, "plain")])
+def test_linear_with_packed_weights(dev, M, N, K, epi):
+    """The weight-stationary kernels fill their registers from W through LDS or, given a copy of W in register
+    order, straight from that: the same registers either way, so the same bytes come out."""
+    from vtpack_amd import ops
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.04).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev) if "bias" in epi else None
+    res = torch.randn(M, N, generator=g).bfloat16().to(dev) if "res" in epi else None
+    act = "gelu" if "gelu" in epi else "none"
+    assert ops.PACK_WEIGHTS
+    packed = ops.packed_weight(w)
+    assert packed is not None and packed.numel() == N * K * 2
+    assert ops.packed_weight(w) is packed                        # made once per tensor and version
+    got = ops.linear(a, w, bias, res, act=act)
+    ops.PACK_WEIGHTS = False
+    try:
+        plain = ops.linear(a, w, bias, res, act=act)
+    finally:
+        ops.PACK_WEIGHTS = True
+    assert torch.equal(got, plain)
+    # a changed weight is packed again
+    w.mul_(2)
+    assert ops.packed_weight(w) is not packed
+    again = ops.linear(a, w, bias, res, act=act)
+    ops.PACK_WEIGHTS = False
+    try:
+        assert torch.equal(again, ops.linear(a, w, bias, res, act=act))
+    finally:
+        ops.PACK_WEIGHTS = True
+
+
+def test_linear_packed_weights_only_where_a_kernel_uses_them(dev):
+    from vtpack_amd import ops, _lib
+    for shape, dtype in (((1000, 192), torch.bfloat16), ((384, 384), torch.float32), ((100, 1536), torch.bfloat16),
+                         ((3456, 384), torch.bfloat16)):
+        w = torch.zeros(shape, dtype=dtype, device=dev)
+        assert ops.packed_weight(w) is None
+    lib = _lib.load()
+    buf = torch.zeros(1000 * 192, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(1000, 192, dtype=torch.bfloat16, device=dev)
+    assert lib.vtdge_linear_prepack(w.data_ptr(), 1000, 192, _lib.BF16, buf.data_ptr(), 0) == _lib.ERR_UNSUPPORTED
+
+
 # ------------------------------------------------------------------ attention / sparse gemm
 def _lengths(seed, B, lo, hi):
     return rng(seed).randint(lo, hi + 1, size=B).astype(np.int64)

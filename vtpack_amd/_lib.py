@@ -15,6 +15,7 @@ CSRC = os.path.join(_PKG, "csrc")
 
 F32, BF16 = 0, 1
 ACT_NONE, ACT_GELU = 0, 1
+ERR_ARG, ERR_UNSUPPORTED, ERR_LAUNCH = -1, -2, -3      # include/vtdge.h
 MAX_SPLITS = 8
 
 _p = ctypes.c_void_p
@@ -33,6 +34,9 @@ SIGNATURES = {
     "vtdge_decompress_layernorm": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_layernorm": [_p, _p, _p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_linear": [_p, _l, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],
+    "vtdge_linear_packed_size": [_i, _i, _i, _p],
+    "vtdge_linear_prepack": [_p, _i, _i, _i, _p, _p],
+    "vtdge_linear_prepacked": [_p, _l, _p, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],
     "vtdge_sparse_attention": [_p, _l, _l, _p, _p, _l, _l, _l, _p, _p, _l, _l, _i, _i, _i, _i, _i, _f, _i, _p],
     "vtdge_batched_sparse_gemm": [_p, _p, _p, _p, _p, _i, _i, _l, _i, _l, _i, _i, _i, _l, _l, _l, _i, _p],
 }

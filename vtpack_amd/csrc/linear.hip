@@ -196,22 +196,91 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
 // weight-stationary variant for bf16, K = 384 (linear_ws.hip)
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
-int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
-                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act, hipStream_t st);
+int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                     int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
+                     hipStream_t st);
 
 // K-split weight-stationary variant for bf16, K = 1536, narrow N (linear_ks.hip)
 bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
-int launch_linear_ks(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
-                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st);
+int launch_linear_ks(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                     int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st);
 
 }  // namespace vtdge
 
 using namespace vtdge;
 
+// ---------------------------------------------------------------------------------------------------------
+// Packed copies of W for the weight-stationary kernels: the 16-byte register images of the MFMA fragments, in the
+// order [column group][wave][fragment][lane], so a wave fills its registers with contiguous 1 KB loads.
+//   layout 1 (K = 384, linear_ws.hip): group = 384 columns; wave w, fragment (j, s), lane (lr, lg) holds
+//            W[384 g + 96 w + 32 j + lr][16 s + 8 lg .. + 7]                       (j < 3, s < 24)
+//   layout 2 (K = 1536, linear_ks.hip): group = 96 columns; wave w, fragment (cb, ks), lane (c16, kg) holds
+//            W[96 g + 16 cb + c16][384 w + 32 ks + 8 kg .. + 7]                    (cb < 6, ks < 12)
+static int packed_layout(int N, int K, int dtype)
+{
+    if (dtype != VTDGE_BF16) return 0;
+    if (K == 384 && N % 384 == 0 && N / 384 <= 8) return 1;
+    if (K == 1536 && N % 96 == 0 && N / 96 <= 8) return 2;
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void linear_prepack_kernel(const bf16_t *__restrict__ W, u32x4 *__restrict__ packed,
+                                                              int N, int K, int layout)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;       // one 16-byte unit each
+    if (idx >= (int64_t)N * K / 8) return;
+    const int lane = (int)(idx & 63);
+    const int f = (int)((idx >> 6) % 72), gw = (int)((idx >> 6) / 72);
+    const int w = gw & 3, g = gw >> 2;
+    int row, k;
+    if (layout == 1) {
+        const int j = f / 24, s = f % 24, lr = lane & 31, lg = lane >> 5;
+        row = 384 * g + 96 * w + 32 * j + lr;
+        k = 16 * s + 8 * lg;
+    } else {
+        const int cb = f / 12, ks = f % 12, c16 = lane & 15, kg = lane >> 4;
+        row = 96 * g + 16 * cb + c16;
+        k = 384 * w + 32 * ks + 8 * kg;
+    }
+    packed[idx] = *reinterpret_cast<const u32x4 *>(W + (int64_t)row * K + k);
+}
+
+extern "C" int vtdge_linear_packed_size(int N, int K, int dtype, int64_t *bytes)
+{
+    VT_REQUIRE(bytes != nullptr, VTDGE_ERR_ARG, "linear_packed_size: NULL result");
+    VT_REQUIRE(N > 0 && K > 0, VTDGE_ERR_ARG, "linear_packed_size: bad sizes N=%d K=%d", N, K);
+    *bytes = packed_layout(N, K, dtype) ? (int64_t)N * K * 2 : 0;
+    return VTDGE_OK;
+}
+
+extern "C" int vtdge_linear_prepack(const void *W, int N, int K, int dtype, void *packed, void *stream)
+{
+    VT_REQUIRE(W && packed, VTDGE_ERR_ARG, "linear_prepack: NULL operand");
+    VT_REQUIRE(N > 0 && K > 0, VTDGE_ERR_ARG, "linear_prepack: bad sizes N=%d K=%d", N, K);
+    const int layout = packed_layout(N, K, dtype);
+    VT_REQUIRE(layout != 0, VTDGE_ERR_UNSUPPORTED, "linear_prepack: no packed layout for N=%d K=%d dtype=%d", N, K,
+               dtype);
+    VT_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)packed & 15) == 0, VTDGE_ERR_ARG,
+               "linear_prepack: W and packed must be 16-byte aligned");
+    const int64_t units = (int64_t)N * K / 8;
+    linear_prepack_kernel<<<(unsigned)ceil_div(units, 256), 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t *)W, (u32x4 *)packed, N, K, layout);
+    return check_launch("linear_prepack");
+}
+
 extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,
                             int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K,
                             int act, int dtype, void *stream)
+{
+    return vtdge_linear_prepacked(A, lda, W, nullptr, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, dtype,
+                                  stream);
+}
+
+extern "C" int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,
+                                      const void *residual, int64_t ldr, void *out, int64_t ldo,
+                                      const int64_t *rows_dev, int64_t rows, int N, int K, int act, int dtype,
+                                      void *stream)
 {
     VT_REQUIRE(A && W && out, VTDGE_ERR_ARG, "linear: NULL operand");
     VT_REQUIRE(dtype == VTDGE_F32 || dtype == VTDGE_BF16, VTDGE_ERR_ARG, "linear: unknown dtype %d", dtype);
@@ -222,14 +291,14 @@ extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const voi
     VT_REQUIRE(((int64_t)K * esz) % 16 == 0 && (lda * esz) % 16 == 0, VTDGE_ERR_UNSUPPORTED,
                "linear: K=%d and lda=%lld must be multiples of %d elements", K, (long long)lda, 16 / esz);
     VT_REQUIRE(lda >= K && ldo >= N && (!residual || ldr >= N), VTDGE_ERR_ARG, "linear: leading dim too small");
-    VT_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, VTDGE_ERR_ARG,
-               "linear: A and W must be 16-byte aligned");
+    VT_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)packed & 15) == 0, VTDGE_ERR_ARG,
+               "linear: A, W and the packed copy of W must be 16-byte aligned");
     if (rows == 0) return VTDGE_OK;
     hipStream_t st = (hipStream_t)stream;
     if (linear_ws_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
-        return launch_linear_ws(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
+        return launch_linear_ws(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
     if (linear_ks_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
-        return launch_linear_ks(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, st);
+        return launch_linear_ks(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, N, st);
     if (linear_dma_applicable(lda, ldr, ldo, N, K, esz, bias, residual, out)) {
         if (dtype == VTDGE_F32)
             return launch_linear_dma<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);

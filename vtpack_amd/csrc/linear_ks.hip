@@ -54,7 +54,7 @@ template <bool HAS_BIAS, bool HAS_RES>
 __global__ __launch_bounds__(256) void linear_ks_kernel(
     const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
     const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
-    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P)
+    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp)
 {
     constexpr int KQ = 768;                  // bytes of a wave's K quarter of a row
     constexpr int KROW = 4 * KQ;             // bytes of a row of W
@@ -75,18 +75,35 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
-    const int64_t M = live_rows(rows_dev, rows);
-    const int M32 = (int)M;
-    const int tiles_m = (M32 + 15) / 16;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int g = slot % groups;                     // column group
     const int p = xcd + 8 * (slot / groups);         // position among the P workgroups of the group
-    const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
-    if (nt == 0) return;
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c16 = lane & 15, kg = lane >> 4;
+
+    // ---- the stationary operand: fragment (cb, ks) = rows 16cb.. of the strip, K step ks of this wave's quarter,
+    // ks < KA in accumulation registers.  Given a copy of W in fragment order (vtdge_linear_prepack: 64 lanes x
+    // 16 B per fragment, contiguous), the registers are loaded straight from it, first thing: nothing here depends
+    // on the row count.
+    u32x4 wfa[CB][KA], wfv[CB][KS - KA];
+    if (Wp != nullptr) {
+        const u32x4 *wp = Wp + ((size_t)(g * 4 + w) * (CB * KS)) * 64 + lane;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const u32x4 v = wp[(cb * KS + ks) * 64];
+                if (ks < KA) wfa[cb][ks] = v;
+                else wfv[cb][ks - KA] = v;
+            }
+    }
+
+    const int64_t M = live_rows(rows_dev, rows);
+    const int M32 = (int)M;
+    const int tiles_m = (M32 + 15) / 16;
+    const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
+    if (nt == 0) return;
     VT_KS_STAMP(0);
 
     // ---- per-lane constants
@@ -130,11 +147,10 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
     auto wrap5 = [](int x) -> int { return x >= RING ? x - RING : x; };          // ring of DH half stages
     auto wrap3 = [](int x) -> int { return x >= 3 * 4096 ? x - 3 * 4096 : x; };  // ring of 3 residual tiles
 
-    // ---- the stationary operand: 12 blocks of 32 W rows x 768 B (block (v, j): rows 32j.. of the strip, K quarter
+    // ---- without a packed copy: 12 blocks of 32 W rows x 768 B (block (v, j): rows 32j.. of the strip, K quarter
     // v) pass through six 24 KB slots; round j brings every wave its j-th block (slots: round 0 -> 0..3;
-    // round 1 -> 4, 5, 0, 1; round 2 -> 2, 3, 4, 5).  Fragment (cb, ks): rows 16cb.. of the strip, K step ks.
-    u32x4 wfa[CB][KA], wfv[CB][KS - KA];
-    {
+    // round 1 -> 4, 5, 0, 1; round 2 -> 2, 3, 4, 5)
+    if (Wp == nullptr) {
         auto issue_w = [&](int v, int j, int lds_slot) {   // this wave's share (6 loads) of block (v, j)
             const uint32_t src = (uint32_t)(g * BN + j * 32) * KROW + v * KQ;
             const uint32_t dst = lds0 + lds_slot * WTILE;
@@ -371,8 +387,8 @@ bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
 }
 
 template <bool HB, bool HR>
-static int go_ks(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr, void *out,
-                 int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
+static int go_ks(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                 int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
 {
     constexpr size_t lds = 4 * 5 * 6144 + 4 * 6 * 1024 + 3 * 4096;   // rings + partial sums + residual ring
     static_assert(lds <= 160 * 1024, "LDS budget");
@@ -392,18 +408,18 @@ static int go_ks(const void *A, int64_t lda, const void *W, const void *bias, co
     if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
     dim3 grid((unsigned)(P * groups)), block(256);
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
-                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P);
+                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp);
     return check_launch("linear");
 }
 
-int launch_linear_ks(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
-                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
+int launch_linear_ks(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                     int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
 {
     const bool hb = bias != nullptr, hr = res != nullptr;
-    if (hb && hr) return go_ks<true, true>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
-    if (hb) return go_ks<true, false>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
-    if (hr) return go_ks<false, true>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
-    return go_ks<false, false>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
+    if (hb && hr) return go_ks<true, true>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
+    if (hb) return go_ks<true, false>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
+    if (hr) return go_ks<false, true>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
+    return go_ks<false, false>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, N, st);
 }
 
 }  // namespace vtdge

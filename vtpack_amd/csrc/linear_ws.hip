@@ -108,7 +108,7 @@ template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES>
 __global__ __launch_bounds__(256) void linear_ws_kernel(
     const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
     const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
-    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P)
+    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp)
 {
     constexpr int KB = KS * 32;                 // bytes of one operand row
     constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
@@ -138,18 +138,35 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
-    const int64_t M = live_rows(rows_dev, rows);
-    const int tiles_m = (int)((M + 31) / 32);
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int g = slot % groups;                     // column group
     const int p = xcd + 8 * (slot / groups);         // position among the P workgroups of the group
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // ---- the stationary operand: fragment (j, s) of this wave's strip of W, s < KA in accumulation registers.
+    // Given a copy of W in fragment order (vtdge_linear_prepack: 64 lanes x 16 B per fragment, contiguous), the
+    // registers are loaded straight from it, first thing: nothing here depends on the row count.
+    u32x4 wfa[NB][KA], wfv[NB][KS - KA];
+    if (Wp != nullptr) {
+        const u32x4 *wp = Wp + ((size_t)(g * 4 + w) * (NB * KS)) * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const u32x4 v = wp[(j * KS + s) * 64];
+                if (s < KA) wfa[j][s] = v;
+                else wfv[j][s - KA] = v;
+            }
+    }
+
+    const int64_t M = live_rows(rows_dev, rows);
+    const int tiles_m = (int)((M + 31) / 32);
     const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
     if (nt == 0) return;
 
     const int M32 = (int)M;
-    const int tid = threadIdx.x, lane = tid & 63;
     VT_WS_STAMP(0);
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lg = lane >> 5;
     const int col0 = g * BN + w * STRIP;             // first output column of this wave
 
@@ -238,8 +255,12 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     // through the six LDS slots.  Round j brings every wave its j-th block, so all four waves read at once; the
     // loads of the next round are in flight meanwhile (slots: round 0 -> 0..3; round 1 -> 4, 5, 0, 1;
     // round 2 -> 2, 3, 4, 5), and the first two tiles of A follow into slots 0 and 1 as soon as those are free.
-    u32x4 wfa[NB][KA], wfv[NB][KS - KA];
-    {
+    if (Wp != nullptr) {
+        // the registers are being loaded from the packed copy: LDS is free and the first tiles of A go out at once
+#pragma unroll
+        for (int k = 0; k < EARLY; k++)
+            if (k < nt) issue_a_all(k);
+    } else {
         // Every workgroup of a column group reads the same 288 KB, and the workgroups of an XCD would walk them in
         // step, all on the same few L2 channels at any moment: each starts its walk somewhere else.
         const int rot = slot % NL, rot4 = (slot / NL) & 3;
@@ -321,7 +342,6 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
 #pragma unroll
     for (int k = EARLY; k < PA; k++)
         if (k < nt) issue_a_all(k);
-
     f32x16 acc[2][NB];
     u32x4 fa[FD + 1];
 
@@ -546,8 +566,8 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
 }
 
 template <int ACT, bool HB, bool HR>
-static int go_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr, void *out,
-                 int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
+static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                 int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
 {
     constexpr int KS = 24, NB = 3;
     constexpr size_t lds = (size_t)6 * 32 * KS * 32;   // six 32-row tiles
@@ -570,15 +590,16 @@ static int go_ws(const void *A, int64_t lda, const void *W, const void *bias, co
     if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
     dim3 grid((unsigned)(P * groups)), block(256);
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
-                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P);
+                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp);
     return check_launch("linear");
 }
 
-int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *bias, const void *res, int64_t ldr,
-                     void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act, hipStream_t st)
+int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                     int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
+                     hipStream_t st)
 {
     const bool hb = bias != nullptr, hr = res != nullptr;
-#define VT_WS(ACT, HB, HR) return go_ws<ACT, HB, HR>(A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, st)
+#define VT_WS(ACT, HB, HR) return go_ws<ACT, HB, HR>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, N, st)
     if (act == VTDGE_ACT_GELU) {
         if (hr) {
             set_error("linear: activation with residual is not built in the weight-stationary kernel");

@@ -5,6 +5,8 @@ raw device pointers plus the current HIP stream to libvtdge.  Row counts of
 packed operands may stay on the device (`rows_dev`), so nothing in this module
 synchronises with the GPU.
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -144,6 +146,33 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     return out
 
 
+PACK_WEIGHTS = True     # module switch (tests compare the two paths)
+
+
+def packed_weight(weight):
+    """The copy of a Linear weight [N, K] in the register order of the weight-stationary kernels, made once per
+    weight tensor and version and kept on the tensor object; None when the kernels for this shape take W as it is."""
+    key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, weight.device)
+    cached = getattr(weight, "_vtdge_packed", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    N, K = weight.shape
+    lib = _lib.load()        # not through call(): these two are no part of a timed step
+    size = ctypes.c_int64(0)
+    if lib.vtdge_linear_packed_size(N, K, dtype_code(weight), ctypes.addressof(size)) != 0:
+        raise _lib.VtdgeError(lib.vtdge_last_error().decode("utf-8", "replace"))
+    packed = None
+    if size.value:
+        packed = torch.empty((size.value,), dtype=torch.uint8, device=weight.device)
+        if lib.vtdge_linear_prepack(ptr(weight), N, K, dtype_code(weight), ptr(packed), stream_ptr()) != 0:
+            raise _lib.VtdgeError(lib.vtdge_last_error().decode("utf-8", "replace"))
+    try:
+        weight._vtdge_packed = (key, packed)
+    except AttributeError:      # an object that takes no attributes: pack again next time
+        pass
+    return packed
+
+
 def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=None):
     """out = act(a @ weight.T + bias) + residual; a [..., K] (last dim contiguous), weight [N, K]."""
     _need_gpu(a, weight, bias, residual)
@@ -162,7 +191,8 @@ def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=N
         r2 = residual.reshape(-1, N)
         if r2.stride(-1) != 1:
             r2 = r2.contiguous()
-    call("vtdge_linear", ptr(a2), a2.stride(0) if rows > 1 else K, ptr(weight), ptr(bias), ptr(r2),
+    packed = packed_weight(weight) if PACK_WEIGHTS and a.dtype == torch.bfloat16 and rows >= 2048 else None
+    call("vtdge_linear_prepacked", ptr(a2), a2.stride(0) if rows > 1 else K, ptr(weight), ptr(packed), ptr(bias), ptr(r2),
          (r2.stride(0) if rows > 1 else N) if r2 is not None else 0, ptr(o2), o2.stride(0) if rows > 1 else N,
          ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr(),
          tag=("linear", act, bias is not None, residual is not None, rows, N, K, rows_dev is not None))
