@@ -80,7 +80,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_compress":
-        return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}>"
+        return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}, {3 if tag[3] * esz // 16 > 64 else 1}>"
     if name == "vtdge_decompress":
         return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
     if name == "vtdge_decompress_layernorm":

@@ -436,18 +436,21 @@ __device__ __forceinline__ void window_sum(const T *__restrict__ base, int W, in
 {
     constexpr int VEC = Elem<T>::VEC;
     if constexpr (SZ > 0) {
-        u32x4 raw[SZ * SZ];
+        // at most eight loads in flight at a time (32 registers); the sum runs over the window in the same order
+        constexpr int NT = SZ * SZ, NBATCH = NT > 8 ? 8 : NT;
 #pragma unroll
-        for (int dy = 0; dy < SZ; dy++)
+        for (int t0 = 0; t0 < NT; t0 += NBATCH) {
+            u32x4 raw[NBATCH];
 #pragma unroll
-            for (int dx = 0; dx < SZ; dx++)
-                raw[dy * SZ + dx] = *reinterpret_cast<const u32x4 *>(base + ((int64_t)dy * W + dx) * C);
+            for (int i = 0; i < NBATCH; i++)
+                raw[i] = *reinterpret_cast<const u32x4 *>(base + ((int64_t)((t0 + i) / SZ) * W + (t0 + i) % SZ) * C);
 #pragma unroll
-        for (int i = 0; i < SZ * SZ; i++) {
-            float f[VEC];
-            Elem<T>::unpack(raw[i], f);
+            for (int i = 0; i < NBATCH; i++) {
+                float f[VEC];
+                Elem<T>::unpack(raw[i], f);
 #pragma unroll
-            for (int c = 0; c < VEC; c++) acc[c] += f[c];
+                for (int c = 0; c < VEC; c++) acc[c] += f[c];
+            }
         }
     } else {
         for (int dy = 0; dy < sz; dy++)
@@ -461,15 +464,18 @@ __device__ __forceinline__ void window_sum(const T *__restrict__ base, int W, in
     }
 }
 
-template <typename T, bool LN, int GS>
-__global__ __launch_bounds__(256) void compress_kernel(const T *__restrict__ x, const int64_t *__restrict__ patches,
+// NIT = 16-byte vectors per lane (1 unless a row is longer than one vector per lane of a 64-lane group).  The
+// one-vector variant is held to 64 registers so that its waves fit next to those of a weight-stationary Linear
+// (one wave per SIMD and most of its registers), which the key/value projection keeps running on every CU meanwhile.
+template <typename T, bool LN, int GS, int NIT>
+__global__ __launch_bounds__(256, NIT == 1 ? 8 : 2) void compress_kernel(const T *__restrict__ x, const int64_t *__restrict__ patches,
                                                         const int64_t *__restrict__ rows_dev, int64_t rows,
                                                         T *__restrict__ out, T *__restrict__ ln_out,
                                                         const T *__restrict__ ln_w, const T *__restrict__ ln_b,
                                                         float eps, int N, int C, int W, int extra)
 {
     constexpr int VEC = Elem<T>::VEC;
-    constexpr int NIT = GS == 64 ? MAX_IT : 1;
+    static_assert(NIT == 1 || GS == 64, "several vectors per lane only with whole-wave groups");
     const int lane = threadIdx.x & (GS - 1);
     const int64_t row = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
     if (row >= live_rows(rows_dev, rows)) return;
@@ -957,14 +963,14 @@ extern "C" int vtdge_compress(const void *x, const int64_t *patches, const int64
     const int gs = group_size(C / vec);
     dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
-#define VT_LAUNCH(T, LNF, GS)                                                                                  \
-    compress_kernel<T, LNF, GS><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out,       \
-                                                        (T *)ln_out, (const T *)ln_weight, (const T *)ln_bias, \
-                                                        ln_eps, N, C, W, extra)
-#define VT_LNF(T, GS) do { if (ln) VT_LAUNCH(T, true, GS); else VT_LAUNCH(T, false, GS); } while (0)
+#define VT_LAUNCH(T, LNF, GS, NIT)                                                                                  \
+    compress_kernel<T, LNF, GS, NIT><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out,       \
+                                                             (T *)ln_out, (const T *)ln_weight, (const T *)ln_bias, \
+                                                             ln_eps, N, C, W, extra)
+#define VT_LNF(T, GS, NIT) do { if (ln) VT_LAUNCH(T, true, GS, NIT); else VT_LAUNCH(T, false, GS, NIT); } while (0)
 #define VT_GROUP(T) \
-    do { if (gs == 64) VT_LNF(T, 64); else if (gs == 32) VT_LNF(T, 32); else if (gs == 16) VT_LNF(T, 16); \
-         else VT_LNF(T, 8); } while (0)
+    do { if (gs == 64) { if (C / vec > WAVE) VT_LNF(T, 64, MAX_IT); else VT_LNF(T, 64, 1); } \
+         else if (gs == 32) VT_LNF(T, 32, 1); else if (gs == 16) VT_LNF(T, 16, 1); else VT_LNF(T, 8, 1); } while (0)
     if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
 #undef VT_GROUP
 #undef VT_LNF
