@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg4|pvt] [--no-graph]
 
 A step is one inference forward of DeiT+DGE over one batch of synthetic images already resident in HBM.
-The headline workload is BASELINE.json's configs[2] ("cfg3": DeiT-S+DGE, 12 layers, bf16, 256 px, batch 256,
-router set for a ~0.5 complexity ratio).  One JSON line is printed:
+The headline workload is "cfg3": DeiT-S+DGE, 12 layers, bf16, 256 px, batch 256, router set for a ~0.5
+complexity ratio (the configuration the images/s metric is quoted on).  One JSON line is printed:
 
   value         images/s over the K timed steps (wall clock between two device synchronisations)
   roofline      the kernel name with the largest share of GPU time: algorithmic flops (or bytes) of its launches
@@ -31,7 +31,7 @@ WORKLOADS = {
     "cfg2": ("deit_dge_s124_tiny_patch16_256", 256, 128, "f32", 3, "DeiT-Ti+DGE 12L fp32 256px B128"),
     "cfg3": ("deit_dge_s124_small_patch16_256", 256, 256, "bf16", 6, "DeiT-S+DGE 12L bf16 256px B256"),
     "cfg5": ("deit_dge_s124_small_patch16_256", 512, 64, "bf16", 6, "DeiT-S+DGE 12L bf16 512px B64"),
-    # the second caller of the path (PVT: four stages, spatially reduced keys/values); not a BASELINE config
+    # the second caller of the path (PVT: four stages, spatially reduced keys/values); not one of the five numbered configurations
     "pvt": ("pvt_dge_s124_small_256", 256, 256, "bf16", (1, 2, 5, 8), "PVT-S+DGE 16L bf16 256px B256"),
 }
 
@@ -387,8 +387,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32, help="images in the CPU baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on one GPU only (the path shards along the batch with no exchange step; "
-              "see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (the path shards along the batch with no exchange step)."
+              " Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():

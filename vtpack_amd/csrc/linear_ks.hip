@@ -148,8 +148,8 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
     auto wrap3 = [](int x) -> int { return x >= 3 * 4096 ? x - 3 * 4096 : x; };  // ring of 3 residual tiles
 
     // ---- without a packed copy: 12 blocks of 32 W rows x 768 B (block (v, j): rows 32j.. of the strip, K quarter
-    // v) pass through six 24 KB slots; round j brings every wave its j-th block (slots: round 0 -> 0..3;
-    // round 1 -> 4, 5, 0, 1; round 2 -> 2, 3, 4, 5)
+    // v) pass through six 24 KB slots; pass j brings every wave its j-th block (slots: pass 0 -> 0..3;
+    // pass 1 -> 4, 5, 0, 1; pass 2 -> 2, 3, 4, 5)
     if (Wp == nullptr) {
         auto issue_w = [&](int v, int j, int lds_slot) {   // this wave's share (6 loads) of block (v, j)
             const uint32_t src = (uint32_t)(g * BN + j * 32) * KROW + v * KQ;
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
         for (int v = 0; v < 4; v++) issue_w(v, 0, v);
         issue_w(0, 1, 4);
         issue_w(1, 1, 5);
-        wait_vmcnt<12>();                      // round 0 has landed
+        wait_vmcnt<12>();                      // pass 0 has landed
         lds_barrier();
         read_w(0, w);
         lds_barrier();                       // slots 0..3 are free
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
         issue_w(3, 1, 1);
         issue_w(0, 2, 2);
         issue_w(1, 2, 3);
-        wait_vmcnt<12>();                      // round 1 has landed
+        wait_vmcnt<12>();                      // pass 1 has landed
         lds_barrier();
         read_w(1, w < 2 ? 4 + w : w - 2);
         lds_barrier();                       // slots 4, 5, 0, 1 are free

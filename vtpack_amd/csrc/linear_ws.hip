@@ -252,9 +252,9 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     };
 
     // ---- the stationary operand: 12 blocks of 32 W rows (block 3 * wave + j holds wave's j-th column block) pass
-    // through the six LDS slots.  Round j brings every wave its j-th block, so all four waves read at once; the
-    // loads of the next round are in flight meanwhile (slots: round 0 -> 0..3; round 1 -> 4, 5, 0, 1;
-    // round 2 -> 2, 3, 4, 5), and the first two tiles of A follow into slots 0 and 1 as soon as those are free.
+    // through the six LDS slots.  Pass j brings every wave its j-th block, so all four waves read at once; the
+    // loads of the next pass are in flight meanwhile (slots: pass 0 -> 0..3; pass 1 -> 4, 5, 0, 1;
+    // pass 2 -> 2, 3, 4, 5), and the first two tiles of A follow into slots 0 and 1 as soon as those are free.
     if (Wp != nullptr) {
         // the registers are being loaded from the packed copy: LDS is free and the first tiles of A go out at once
 #pragma unroll
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         issue_w(0, 1, 4);
         issue_w(1, 1, 5);
         VT_WS_STAMP(40);
-        wait_vmcnt<2 * NL>();                  // round 0 has landed
+        wait_vmcnt<2 * NL>();                  // pass 0 has landed
         VT_WS_STAMP(41);
         lds_barrier();
         // the bias values are consumed here as far as the compiler is concerned: their loads are issued above and
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         issue_w(0, 2, 2);
         issue_w(1, 2, 3);
         VT_WS_STAMP(43);
-        wait_vmcnt<2 * NL>();                  // round 1 has landed
+        wait_vmcnt<2 * NL>();                  // pass 1 has landed
         VT_WS_STAMP(44);
         lds_barrier();
         read_w(1, w < 2 ? 4 + w : w - 2);
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         for (int k = 0; k < EARLY; k++)
             if (k < nt) issue_a_all(k);
         VT_WS_STAMP(46);
-        wait_vmcnt_dyn(issued);                // round 2 has landed (all but the tiles of A)
+        wait_vmcnt_dyn(issued);                // pass 2 has landed (all but the tiles of A)
         VT_WS_STAMP(47);
         lds_barrier();
         read_w(2, 2 + w);
