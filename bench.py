@@ -9,7 +9,8 @@ complexity ratio (the configuration the images/s metric is quoted on).  One JSON
 
   value         images/s over the K timed steps (wall clock between two device synchronisations)
   roofline      the kernel name with the largest share of GPU time: algorithmic flops (or bytes) of its launches
-                divided by their HIP-event durations, against MI355X's published peak
+                divided by their HIP-event durations, against MI355X's published peak; a matrix kernel is priced
+                against both roofs and reported against the one it is nearer to (the other under "other_roof")
   kernels       the same figures for every libvtdge kernel of the step
   cpu_baseline  the torch-CPU restatement of the same model (oracle/torch_ref.py) timed on this box's host cores
                 on a bounded sample of the same workload
@@ -121,11 +122,13 @@ def algorithmic_work(name, tag, esz, geo):
     geo: dict with B, N, C, L (live packed rows), regions and extra of the block the launch belongs to."""
     B, N, C, L = geo["B"], geo["N"], geo["C"], geo["L"]
     if name in ("vtdge_linear", "vtdge_linear_prepacked"):
-        _, _, _, _, rows, Nn, K, packed = tag
+        _, _, _, has_res, rows, Nn, K, packed = tag
         M = L if packed else rows
-        return "mfma", 2.0 * M * Nn * K
+        # operands once: A, W, the output and, when there is one, the residual
+        return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn * (2 if has_res else 1)) * esz
     if name == "vtdge_sparse_attention":
-        return "mfma", 4.0 * L * tag[4] * C               # tag[4] = keys per sample
+        # tag[4] = keys per sample; bytes: q in, out, every sample's K and V once
+        return "mfma", 4.0 * L * tag[4] * C, (2 * L * C + 2 * B * tag[4] * C) * esz
     if name == "vtdge_compress":
         # read every token once, the descriptors, write every query once (+ the fused LayerNorm copy)
         return "hbm", B * N * C * esz + 32 * L + L * C * esz * (2 if tag[1] else 1)
@@ -246,16 +249,32 @@ def run_model_workload(args, torch):
             blk = 0
         # a block's launches end with its scatter; what precedes block 0 or follows the last block is dense
         geo = dict(geos[min(blk, len(blocks) - 1)], L=lens[i // per_step][min(blk, len(blocks) - 1)])
-        bound, amount = algorithmic_work(name, tag, esz, geo)
+        bound, amount, *rest = algorithmic_work(name, tag, esz, geo)
         sym = kernel_symbol(name, tag, dt)
-        st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0})
+        st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0, "bytes": 0.0})
         st["launches"] += 1
         st["seconds"] += sec
         st["work"] += amount
+        st["bytes"] += rest[0] if rest else 0.0
         if name == "vtdge_decompress":
             blk += 1
     kernels = {}
     for sym, st in stats.items():
+        # A matrix kernel is priced against both roofs (the K = 384 and narrow-N GEMMs of this model sit near the
+        # ridge, attention below it): the one it is nearer to is the one that binds, and the other is kept beside it.
+        other = None
+        if st["bound"] == "mfma" and st["bytes"] > 0:
+            f_m = st["work"] / st["seconds"] / 1e12 / PEAK["mfma"][dt]
+            f_h = st["bytes"] / st["seconds"] / 1e9 / PEAK["hbm"]
+            if f_h > f_m:
+                other = {"bound": "mfma", "achieved": round(st["work"] / st["seconds"] / 1e12, 2),
+                         "peak": PEAK["mfma"][dt], "unit": "TFLOP/s", "frac": round(f_m, 4),
+                         "algorithmic_per_launch": int(st["work"] / st["launches"])}
+                st["bound"], st["work"] = "hbm", st["bytes"]
+            else:
+                other = {"bound": "hbm", "achieved": round(st["bytes"] / st["seconds"] / 1e9, 2), "peak": PEAK["hbm"],
+                         "unit": "GB/s", "frac": round(f_h, 4),
+                         "algorithmic_per_launch": int(st["bytes"] / st["launches"])}
         peak = PEAK["hbm"] if st["bound"] == "hbm" else PEAK["mfma"][dt]
         unit = "GB/s" if st["bound"] == "hbm" else "TFLOP/s"
         ach = st["work"] / st["seconds"] / (1e9 if st["bound"] == "hbm" else 1e12)
@@ -263,6 +282,8 @@ def run_model_workload(args, torch):
                         "frac": round(ach / peak, 4), "avg_us": round(st["seconds"] / st["launches"] * 1e6, 2),
                         "launches_per_step": st["launches"] // inst_steps,
                         "share": 0.0}
+        if other is not None:
+            kernels[sym]["other_roof"] = other
     tot = sum(st["seconds"] for st in stats.values())
     for sym, st in stats.items():
         kernels[sym]["share"] = round(st["seconds"] / tot, 4)
@@ -273,6 +294,8 @@ def run_model_workload(args, torch):
         kernels[sym]["algorithmic_per_launch"] = int(stats[sym]["work"] / stats[sym]["launches"])
         kernels[sym]["traffic"] = traffic.get(sym)
     roof.update({"kernel": dom, "avg_us": kernels[dom]["avg_us"], "traffic": traffic.get(dom)})
+    if "other_roof" in kernels[dom]:
+        roof["other_roof"] = kernels[dom]["other_roof"]
 
     # one plain device-to-device copy of known size (256 MiB), so that a counter run of this script carries its
     # own yardstick for the HBM byte counters
