@@ -165,10 +165,20 @@ def block_forward(sd, prefix, x, num_heads, gate=None, indices=None, eps=1e-6, t
 
 
 def deit_dge_forward(sd, images, num_heads, depth, patch=16, eps=1e-6, forced_indices=None, traces=None):
-    """vtpack/models/dge/deit_dge.py:267-299 (cls token, no distillation).  images [B,3,S,S] -> logits."""
+    """vtpack/models/dge/deit_dge.py:267-299 at inference.  images [B,3,S,S] -> logits.
+
+    The variant is read off the state dict, as the reference's constructor fixes it (deit_dge.py:179-214):
+    `cls_token` absent -> no extra token and the head sees the token mean; `dist_token` present -> two extra tokens
+    and the mean of `head` and `head_dist`; `pre_logits.fc.*` present -> Linear + tanh before the head."""
     x = F.conv2d(images, sd["patch_embed.proj.weight"], sd["patch_embed.proj.bias"], stride=patch)
     x = x.flatten(2).transpose(1, 2)
-    x = torch.cat((sd["cls_token"].expand(x.shape[0], -1, -1), x), dim=1) + sd["pos_embed"]
+    B = x.shape[0]
+    if "cls_token" in sd:
+        front = [sd["cls_token"].expand(B, -1, -1)]
+        if "dist_token" in sd:
+            front.append(sd["dist_token"].expand(B, -1, -1))
+        x = torch.cat(front + [x], dim=1)
+    x = x + sd["pos_embed"]
     for i in range(depth):
         tr = {} if traces is not None else None
         x = block_forward(sd, f"blocks.{i}.", x, num_heads, eps=eps, trace=tr,
@@ -176,8 +186,16 @@ def deit_dge_forward(sd, images, num_heads, depth, patch=16, eps=1e-6, forced_in
         if traces is not None:
             traces.append(tr)
     C = x.shape[-1]
-    x = F.layer_norm(x, (C,), sd["norm.weight"], sd["norm.bias"], eps)[:, 0]
-    return F.linear(x, sd["head.weight"], sd["head.bias"])
+    x = F.layer_norm(x, (C,), sd["norm.weight"], sd["norm.bias"], eps)
+    head = lambda name, t: F.linear(t, sd[name + ".weight"], sd[name + ".bias"]) if name + ".weight" in sd else t  # noqa: E731
+    if "cls_token" not in sd:
+        return head("head", x.mean(dim=1))
+    if "dist_token" in sd:
+        return (head("head", x[:, 0]) + head("head_dist", x[:, 1])) / 2
+    x = x[:, 0]
+    if "pre_logits.fc.weight" in sd:
+        x = torch.tanh(F.linear(x, sd["pre_logits.fc.weight"], sd["pre_logits.fc.bias"]))
+    return head("head", x)
 
 
 def pvt_dge_forward(sd, images, num_heads, depths, sr_ratios, patch=4, eps=1e-6, embed_eps=1e-5, forced_indices=None,

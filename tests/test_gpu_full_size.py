@@ -1,5 +1,6 @@
-"""The headline configuration at its full size (DeiT-S+DGE, bf16, batch 256, 256 px: 65 792 tokens of 384 channels,
-about 27 000 packed queries per layer), where the CPU oracle would take minutes: every kernel of the path is
+"""The headline configuration (DeiT-S+DGE, bf16, batch 256, 256 px: 65 792 tokens of 384 channels, about 27 000
+packed queries per layer) and the high-resolution one (batch 64, 512 px: 1025 tokens and 64 regions per sample, key
+/ value length 1025) at their full sizes, where the CPU oracle would take minutes: every kernel of the path is
 checked through properties that hold at any size and whose expected values are exact."""
 import numpy as np
 import pytest
@@ -9,13 +10,22 @@ from util import random_indices
 
 pytestmark = pytest.mark.gpu
 
-B, H, W, C, R, EXTRA, HEADS = 256, 16, 16, 384, 4, 1, 6
-N = EXTRA + H * W
+C, R, EXTRA, HEADS = 384, 4, 1, 6
 SPLITS = [4, 2, 1]
+B = H = W = N = IMG = 0      # set per configuration by the fixture below
+
+
+@pytest.fixture(scope="module", params=["b256_256px", "b64_512px"], autouse=True)
+def geometry(request):
+    global B, H, W, N, IMG
+    B, H, IMG = (256, 16, 256) if request.param == "b256_256px" else (64, 32, 512)
+    W = H
+    N = EXTRA + H * W
+    return request.param
 
 
 @pytest.fixture(scope="module")
-def routed(dev):
+def routed(dev, geometry):
     """Gate indices with the mix the benchmark's router produces, and their packed descriptors."""
     from vtpack_amd import ops
     idx = torch.from_numpy(random_indices(5, B, H // R, W // R, p=[0.1, 0.25, 0.65])).to(dev)
@@ -25,10 +35,10 @@ def routed(dev):
 
 
 def test_descriptors_partition_every_sample(routed):
-    """Rows sorted by sample, extra tokens first; the windows of a sample tile its 16 x 16 grid exactly once;
+    """Rows sorted by sample, extra tokens first; the windows of a sample tile its token grid exactly once;
     lengths and offsets follow from the gate indices in closed form."""
     idx, splits, patches, offsets, lengths = routed
-    ps = splits[idx]                                            # [B, 4, 4]
+    ps = splits[idx]                                            # [B, Hr, Wr]
     want_len = EXTRA + (ps * ps).sum(dim=(1, 2))
     assert torch.equal(lengths, want_len)
     assert torch.equal(offsets, torch.cat([torch.zeros(1, dtype=torch.int64, device=idx.device), want_len.cumsum(0)]))
@@ -80,12 +90,12 @@ def test_compress_inverts_scatter(dev, routed):
 
 def test_router_picks_the_planted_split(dev):
     """Channel s of every token is set from the split planted for its region and the gate weight reads exactly
-    that channel: the router returns the planted split for all 4096 regions."""
+    that channel: the router returns the planted split for every region of the batch."""
     from vtpack_amd import ops
     want = torch.from_numpy(random_indices(9, B, H // R, W // R)).to(dev)
     x = torch.zeros(B, N, C, dtype=torch.bfloat16, device=dev)
-    onehot = torch.nn.functional.one_hot(want, 3).to(torch.bfloat16)               # [B, 4, 4, 3]
-    grid = onehot.repeat_interleave(R, dim=1).repeat_interleave(R, dim=2)             # [B, 16, 16, 3]
+    onehot = torch.nn.functional.one_hot(want, 3).to(torch.bfloat16)               # [B, Hr, Wr, 3]
+    grid = onehot.repeat_interleave(R, dim=1).repeat_interleave(R, dim=2)             # [B, H, W, 3]
     x[:, EXTRA:, :3] = grid.reshape(B, H * W, 3)
     x[:, :EXTRA] = 7.0                                                                # extra tokens are not pooled
     wgt = torch.zeros(3, C, dtype=torch.bfloat16, device=dev)
@@ -102,7 +112,7 @@ def test_linear_with_selector_weights_is_exact(dev):
     documented order."""
     from vtpack_amd import ops
     g = torch.Generator().manual_seed(3)
-    L = 27001
+    L = 27001 if H == 16 else 28703
     a = torch.randn(L, C, generator=g).bfloat16().to(dev)
     eye = torch.eye(C, dtype=torch.bfloat16, device=dev)
     assert torch.equal(ops.linear(a, eye), a)                                          # q / proj shape
@@ -148,25 +158,25 @@ def test_attention_of_constant_values_and_sample_isolation(dev, routed):
     assert not torch.equal(again[~even], base[~even])
 
 
-def test_model_batch_of_256_is_64_samples_four_times(dev):
-    """The whole forward at the headline batch: samples do not see each other, so the logits of the first 64 images
-    are the logits of those 64 images run alone (same kernels on both sides: each run has well over 2048 packed
+def test_model_batch_is_its_first_quarter_four_times(dev):
+    """The whole forward at the full batch: samples do not see each other, so the logits of the first quarter of the
+    images are the logits of those images run alone (same kernels on both sides: each run has well over 2048 packed
     rows per layer), and a second run of the batch returns the same bits."""
     from vtpack_amd.models import dge as zoo
     from vtpack_amd.synthetic import set_synthetic_router, synthetic_images
     torch.manual_seed(0)
-    m = zoo.deit_dge_s124_small_patch16_256(img_size=256)
+    m = zoo.deit_dge_s124_small_patch16_256(img_size=IMG)
     set_synthetic_router(m, 0)
     m = m.eval().to(dev).to(torch.bfloat16)
-    img = synthetic_images(B, 256, seed=0, dtype=torch.bfloat16, device=dev)
+    img = synthetic_images(B, IMG, seed=0, dtype=torch.bfloat16, device=dev)
     with torch.no_grad():
         full = m(img)
         lens = [blk.dge.states["batches_device"].clone() for blk in m.blocks]
         again = m(img)
-        part = m(img[:64].contiguous())
+        part = m(img[:B // 4].contiguous())
     assert full.shape == (B, 1000) and bool(torch.isfinite(full.float()).all())
     assert torch.equal(full, again)
-    assert torch.equal(full[:64], part)
+    assert torch.equal(full[:B // 4], part)
     # the router really mixes grains at this size: between a third and two thirds of the tokens stay queries
     ratio = float(sum(int(l.sum()) for l in lens)) / (len(lens) * B * N)
     assert 0.3 < ratio < 0.7

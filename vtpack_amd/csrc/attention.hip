@@ -233,15 +233,7 @@ static int launch_attention(const void *q, int64_t q_rs, int64_t q_hs, const voi
     const size_t lds = (size_t)KSTAGE * (D * ESZ + 16) + (size_t)D * (KSTAGE * ESZ + 16);
     const int qchunks = (int)ceil_div(max_rows, QROWS);
     auto kern = sparse_attention_kernel<T, D>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            set_error("sparse_attention: cannot reserve %zu bytes of LDS", lds);
-            return VTDGE_ERR_LAUNCH;
-        }
-        attr_done = true;
-    }
+    VT_RESERVE_LDS(kern, lds, "sparse_attention");
     dim3 grid((unsigned)((int64_t)B * qchunks), (unsigned)h), block(256);
     kern<<<grid, block, lds, st>>>((const T *)q, q_rs, q_hs, (const T *)k, (const T *)v, kv_bs, kv_ts, kv_hs, offsets,
                                    (T *)out, o_rs, o_hs, n, qchunks, scale);

@@ -227,11 +227,11 @@ __device__ __forceinline__ void attn_stage_resident_nb(int nb, const unsigned ch
 __global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_resident_kernel(
     const bf16_t *__restrict__ q, int64_t q_rs, int64_t q_hs, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, int64_t kv_bs, int64_t kv_ts, int64_t kv_hs, const int64_t *__restrict__ offsets,
-    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale, int B, int h, int order)
+    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale, int B, int h)
 {
     constexpr int MAXV = 9;          // 16-byte V chunks per thread: covers n_pad = 288
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int b = order ? blockIdx.x / h : blockIdx.x % B, head = order ? blockIdx.x % h : blockIdx.x / B;
+    const int b = blockIdx.x % B, head = blockIdx.x / B;
     const int64_t row0 = offsets[b];
     const int Lb = (int)(offsets[b + 1] - row0);
     if (Lb <= 0) return;
@@ -455,38 +455,16 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
         const int npad = (n + 31) & ~31;
         const size_t lds_r = (size_t)npad * 128 + 64 * ((size_t)((n + 63) & ~63) * 2 + 16);
         auto kern_r = sparse_attention_bf16_d64_resident_kernel;
-        static bool attr_r = false;
-        if (!attr_r) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern_r), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    80 * 1024) != hipSuccess) {
-                set_error("sparse_attention: cannot reserve LDS");
-                return VTDGE_ERR_LAUNCH;
-            }
-            attr_r = true;
-        }
-        static int order = -1;
-        if (order < 0) {
-            const char *e = getenv("VTDGE_ATT_ORDER");
-            order = e ? atoi(e) : 0;
-        }
+        VT_RESERVE_LDS(kern_r, 80 * 1024, "sparse_attention");
         dim3 grid_r((unsigned)(B * h)), block_r(256);
         kern_r<<<grid_r, block_r, lds_r, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v,
-                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale, B, h,
-                                               order);
+                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale, B, h);
         return check_launch("sparse_attention");
     }
     const size_t lds = 2 * (size_t)ABUF;
     const int qchunks = (int)ceil_div(max_rows, AQ);
     auto kern = sparse_attention_bf16_d64_kernel;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            set_error("sparse_attention: cannot reserve %zu bytes of LDS", lds);
-            return VTDGE_ERR_LAUNCH;
-        }
-        attr_done = true;
-    }
+    VT_RESERVE_LDS(kern, lds, "sparse_attention");
     dim3 grid((unsigned)((int64_t)B * qchunks), (unsigned)h), block(256);
     kern<<<grid, block, lds, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v, kv_bs, kv_ts,
                                    kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, qchunks, scale);

@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <mutex>
 #include <utility>
 
 #include "../../include/vtdge.h"
@@ -20,6 +21,22 @@ int check_launch(const char *what);
             set_error(__VA_ARGS__);  \
             return (code);           \
         }                            \
+    } while (0)
+
+// Raises a kernel's dynamic-LDS limit the first time its call site runs (once per template instantiation, safe
+// when several host threads make their first call at the same time).
+#define VT_RESERVE_LDS(kern, bytes, what)                                                                       \
+    do {                                                                                                        \
+        static std::once_flag vt_once;                                                                          \
+        static hipError_t vt_err = hipSuccess;                                                                  \
+        std::call_once(vt_once, [&] {                                                                           \
+            vt_err = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes));             \
+        });                                                                                                     \
+        if (vt_err != hipSuccess) {                                                                             \
+            ::vtdge::set_error("%s: cannot reserve %zu bytes of LDS", what, (size_t)(bytes));                   \
+            return VTDGE_ERR_LAUNCH;                                                                            \
+        }                                                                                                       \
     } while (0)
 
 // ---------------------------------------------------------------- types

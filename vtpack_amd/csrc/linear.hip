@@ -157,15 +157,7 @@ static int launch_linear(const void *A, int64_t lda, const void *W, const void *
 #define VT_GO(ACT, HB, HR)                                                                                      \
     do {                                                                                                        \
         auto kern = linear_kernel<T, ACT, HB, HR>;                                                              \
-        static bool attr_done = false; /* one flag per instantiation */                                         \
-        if (!attr_done) {                                                                                       \
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                       \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {      \
-                set_error("linear: cannot reserve %zu bytes of LDS", lds);                                      \
-                return VTDGE_ERR_LAUNCH;                                                                        \
-            }                                                                                                   \
-            attr_done = true;                                                                                   \
-        }                                                                                                       \
+        VT_RESERVE_LDS(kern, lds, "linear");                                                                    \
         kern<<<grid, block, lds, st>>>((const T *)A, lda, (const T *)W, (const T *)bias, (const T *)res, ldr,   \
                                        (T *)out, ldo, rows_dev, rows, N, K);                                    \
     } while (0)

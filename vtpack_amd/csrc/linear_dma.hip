@@ -286,15 +286,7 @@ static int go(const LinArgs &a)
     static_assert(lds <= 160 * 1024, "LDS budget");
     constexpr int WGS_PER_CU = lds <= 80 * 1024 ? 2 : 1;
     auto kern = linear_dma_kernel<T, BM, BN, WGM, WGN, NWP, ACT, HB, HR, NSTAGE, LATE>;
-    static bool attr_done = false;  // one flag per instantiation
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            set_error("linear: cannot reserve %zu bytes of LDS", lds);
-            return VTDGE_ERR_LAUNCH;
-        }
-        attr_done = true;
-    }
+    VT_RESERVE_LDS(kern, lds, "linear");
     // persistent grid: what fits on the 256 CUs at once, but never more workgroups than tiles per XCD
     const int64_t tiles_per_xcd = ceil_div(ceil_div(a.rows, BM), 8) * ceil_div(a.N, BN);
     int64_t wgs_per_xcd = 32 * WGS_PER_CU;
@@ -321,16 +313,6 @@ static int pick_epilogue(const LinArgs &a)
     return go<T, BM, BN, WGM, WGN, NWP, VTDGE_ACT_NONE, false, false>(a);
 }
 
-static int tuning_override()
-{
-    static int v = -2;
-    if (v == -2) {
-        const char *e = getenv("VTDGE_LINEAR_CFG");
-        v = e ? atoi(e) : -1;
-    }
-    return v;
-}
-
 // Whether the pipelined kernel can take the problem (the generic kernel takes the rest).
 bool linear_dma_applicable(int64_t lda, int64_t ldr, int64_t ldo, int N, int K, int esz, const void *bias,
                            const void *res, const void *out)
@@ -346,21 +328,10 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
                       hipStream_t st)
 {
     LinArgs a{A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, K, act, st};
-    int cfg = tuning_override();
-    if (cfg < 0) {
-        // wide outputs: 256x128 tiles on 8 MFMA waves; narrow ones (N <= 512): 128x128 on 4, for more tiles
-        // (128x384 tiles, whole rows of a narrow output on a two-stage ring, measured no faster: override 6)
-        cfg = N >= 768 ? 0 : 1;
-    }
-    switch (cfg) {
-    case 0: return pick_epilogue<T, 256, 128, 4, 2, 4>(a);
-    case 1: return pick_epilogue<T, 128, 128, 2, 2, 4>(a);
-    case 2: return pick_epilogue<T, 256, 128, 4, 2, 2>(a);
-    case 3: return pick_epilogue<T, 256, 128, 2, 2, 4>(a);
-    case 4: return pick_epilogue<T, 128, 128, 4, 2, 4>(a);
-    case 6: return pick_epilogue<T, 128, 384, 2, 4, 4>(a);
-    default: return pick_epilogue<T, 128, 256, 2, 4, 4>(a);
-    }
+    // wide outputs: 256x128 tiles on 8 MFMA waves; narrow ones (N <= 512): 128x128 on 4, for more tiles.  Other
+    // shapes of the same template (2 loader waves, 128x256 and 128x384 tiles on a two-stage ring) measured no faster.
+    if (N >= 768) return pick_epilogue<T, 256, 128, 4, 2, 4>(a);
+    return pick_epilogue<T, 128, 128, 2, 2, 4>(a);
 }
 
 template int launch_linear_dma<float>(const void *, int64_t, const void *, const void *, const void *, int64_t, void *,

@@ -25,17 +25,6 @@
 
 namespace vtdge {
 
-#ifdef VT_KS_DEBUG
-__device__ long long ks_dbg[4][256];
-#define VT_KS_STAMP(i)                                                                         \
-    do {                                                                                       \
-        if (lane == 0 && blockIdx.x == 0 && (i) < 256) ks_dbg[w][(i)] = clock64();             \
-    } while (0)
-#else
-#define VT_KS_STAMP(i) do { } while (0)
-#endif
-
-
 // D = W_frag * A_frag^T (+ D) on 16 x 16 x 32; the stationary fragment in accumulation (A) or vector (V) registers;
 // Z starts a new sum.
 __device__ __forceinline__ void mma16_a(f32x4 &d, const u32x4 &wfrag, const u32x4 &afrag)
@@ -104,7 +93,6 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
     const int tiles_m = (M32 + 15) / 16;
     const int nt = tiles_m > p ? (tiles_m - p + P - 1) / P : 0;
     if (nt == 0) return;
-    VT_KS_STAMP(0);
 
     // ---- per-lane constants
     // fragment reads (16 rows x 4 chunks of a 128-byte slab): row c16, chunk (4p + kg) ^ ((c16/2)%8), p = K step % 2
@@ -196,7 +184,6 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
         lds_barrier();                       // LDS is free
     }
 
-    VT_KS_STAMP(1);
     // ---- prologue: this wave's rows of residual tile 0, then half stages 0..3 (tiles 0, 1).  Tiles past this workgroup's
     // last one are loaded all the same (their rows are clamped into the matrix) and never used: no load in this
     // kernel is conditional, so the number of operations in flight at any point is known at compile time.
@@ -277,9 +264,7 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
     auto tile_step = [&](auto pp_tag, auto epi_tag, int k) {
         constexpr int PP = decltype(pp_tag)::value;
         constexpr bool EPI = decltype(epi_tag)::value;
-        VT_KS_STAMP(4 + 4 * k);
         wait_vmcnt<12>();                     // this wave's loads of tile k and of the residual of tile k have landed
-        VT_KS_STAMP(5 + 4 * k);
         const int cs0 = fresh(cs16);
         const int o0 = hb, o1 = wrap5(hb + HS), o4 = wrap5(hb + 4 * HS);   // half stages 2k (and 2k+5), 2k+1, 2k+4
         hb = wrap5(hb + 2 * HS);
@@ -330,11 +315,9 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (EPI && s == 5) {
-                VT_KS_STAMP(6 + 4 * k);
                 // LDS operations complete in order and three fragment reads were issued after the last write
                 asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");
                 block_barrier();                         // the partial sums of tile k-1 are visible
-                VT_KS_STAMP(7 + 4 * k);
             }
         });
         if constexpr (EPI) block_barrier();              // every wave has read the partial sums of tile k-1
@@ -374,12 +357,6 @@ __global__ __launch_bounds__(256) void linear_ks_kernel(
 bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out)
 {
-    static int off = -1;   // VTDGE_LINEAR_KS=0 keeps these shapes on the streaming kernel (A/B timing)
-    if (off < 0) {
-        const char *e = getenv("VTDGE_LINEAR_KS");
-        off = (e && atoi(e) == 0) ? 1 : 0;
-    }
-    if (off) return false;
     return esz == 2 && K == 1536 && act == VTDGE_ACT_NONE && N % 96 == 0 && N / 96 <= 8 && rows >= 2048 &&
            rows * lda < (1ll << 31) && (res == nullptr || rows * ldr < (1ll << 31)) && ldo < (1ll << 31) &&
            lda % 8 == 0 && ldo % 4 == 0 && (res == nullptr || ldr % 8 == 0) &&
@@ -393,15 +370,7 @@ static int go_ks(const void *A, int64_t lda, const void *W, const void *Wp, cons
     constexpr size_t lds = 4 * 5 * 6144 + 4 * 6 * 1024 + 3 * 4096;   // rings + partial sums + residual ring
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = linear_ks_kernel<HB, HR>;
-    static bool attr_done = false;  // one flag per instantiation
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            set_error("linear: cannot reserve %zu bytes of LDS", lds);
-            return VTDGE_ERR_LAUNCH;
-        }
-        attr_done = true;
-    }
+    VT_RESERVE_LDS(kern, lds, "linear");
     const int groups = N / 96;
     int P = (256 / groups) & ~7;
     const int64_t tiles_m = ceil_div(rows, 16);

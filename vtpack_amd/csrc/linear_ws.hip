@@ -34,17 +34,6 @@
 
 namespace vtdge {
 
-#ifdef VT_WS_DEBUG
-__device__ long long ws_dbg[4][64];
-#define VT_WS_STAMP(i)                                                                         \
-    do {                                                                                       \
-        if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100) && (i) < 64)                     \
-            ws_dbg[blockIdx.x == 0 ? 0 : 1][(i)] = clock64();                                  \
-    } while (0)
-#else
-#define VT_WS_STAMP(i) do { } while (0)
-#endif
-
 // D = W_frag * A_frag^T (+ D).  The stationary fragment sits in accumulation registers (A) or vector registers (V);
 // Z starts a new sum.  Issued from assembly so the register classes are exactly these.
 __device__ __forceinline__ void mma_a(f32x16 &d, const u32x4 &wfrag, const u32x4 &afrag)
@@ -166,7 +155,6 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     if (nt == 0) return;
 
     const int M32 = (int)M;
-    VT_WS_STAMP(0);
     const int lr = lane & 31, lg = lane >> 5;
     const int col0 = g * BN + w * STRIP;             // first output column of this wave
 
@@ -288,42 +276,32 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         for (int v = 0; v < 4; v++) issue_w((v + rot4) & 3, 0, (v + rot4) & 3);
         issue_w(0, 1, 4);
         issue_w(1, 1, 5);
-        VT_WS_STAMP(40);
         wait_vmcnt<2 * NL>();                  // pass 0 has landed
-        VT_WS_STAMP(41);
         lds_barrier();
         // the bias values are consumed here as far as the compiler is concerned: their loads are issued above and
         // waited for now, not next to their first real use in the middle of the pipeline
 #pragma unroll
         for (int j = 0; j < NB; j++) asm volatile("" : "+v"(wb[j]));
         read_w(0, w);
-        VT_WS_STAMP(42);
         lds_barrier();                       // slots 0..3 are free
         issue_w(2, 1, 0);
         issue_w(3, 1, 1);
         issue_w(0, 2, 2);
         issue_w(1, 2, 3);
-        VT_WS_STAMP(43);
         wait_vmcnt<2 * NL>();                  // pass 1 has landed
-        VT_WS_STAMP(44);
         lds_barrier();
         read_w(1, w < 2 ? 4 + w : w - 2);
-        VT_WS_STAMP(45);
         lds_barrier();                       // slots 4, 5, 0, 1 are free
         issue_w(2, 2, 4);
         issue_w(3, 2, 5);
 #pragma unroll
         for (int k = 0; k < EARLY; k++)
             if (k < nt) issue_a_all(k);
-        VT_WS_STAMP(46);
         wait_vmcnt_dyn(issued);                // pass 2 has landed (all but the tiles of A)
-        VT_WS_STAMP(47);
         lds_barrier();
         read_w(2, 2 + w);
-        VT_WS_STAMP(48);
         lds_barrier();                       // slots 2..5 are free
     }
-    VT_WS_STAMP(1);
     // ---- rest of the prologue: first residual tiles, remaining first tiles of A
     if constexpr (HAS_RES) {
 #pragma unroll
@@ -406,9 +384,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         constexpr bool EPI = decltype(epi_tag)::value;
         using PQ = std::integral_constant<int, 1 - PP>;
         const bool more = k + 1 < nt;
-        VT_WS_STAMP(3 + 2 * k);
         wait_step(k);
-        VT_WS_STAMP(4 + 2 * k);
         block_barrier();   // what was awaited is in LDS for every wave; the slots read last step are free
 
         // Direct loads of this step: the residual of tile k+PR and A(k+PA), six each per wave.  The waves take turns
@@ -520,7 +496,6 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
 #pragma unroll
         for (int s = 0; s < FD; s++) fa[s] = *reinterpret_cast<const u32x4 *>(smem + (s >> 2) * 4096 + cs[s & 3]);
     }
-    VT_WS_STAMP(2);
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     tile_step(I0{}, std::false_type{}, 0);
@@ -530,7 +505,6 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         tile_step(I0{}, std::true_type{}, k + 1);
     }
     if (k < nt) tile_step(I1{}, std::true_type{}, k);
-    VT_WS_STAMP(3 + 2 * nt);
     // ---- last tile's epilogue
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs' results must have reached the registers
     unsigned char *orow = out_row(nt - 1);
@@ -544,19 +518,12 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         epi_part2(n);
         epi_part3(n, orow);
     }
-    VT_WS_STAMP(4 + 2 * nt);
 }
 
 // ----------------------------------------------------------------------------- host
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out)
 {
-    static int off = -1;   // VTDGE_LINEAR_WS=0 keeps these shapes on the streaming kernel (A/B timing)
-    if (off < 0) {
-        const char *e = getenv("VTDGE_LINEAR_WS");
-        off = (e && atoi(e) == 0) ? 1 : 0;
-    }
-    if (off) return false;
     // the residual is added inside the accumulator, i.e. before an activation: such a pair goes elsewhere
     if (res != nullptr && act != VTDGE_ACT_NONE) return false;
     return esz == 2 && K == 384 && lda < (1ll << 31) && ldo < (1ll << 31) && ldr < (1ll << 31) && N % 384 == 0 &&
@@ -573,15 +540,7 @@ static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, cons
     constexpr size_t lds = (size_t)6 * 32 * KS * 32;   // six 32-row tiles
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR>;
-    static bool attr_done = false;  // one flag per instantiation
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            set_error("linear: cannot reserve %zu bytes of LDS", lds);
-            return VTDGE_ERR_LAUNCH;
-        }
-        attr_done = true;
-    }
+    VT_RESERVE_LDS(kern, lds, "linear");
     const int groups = N / (4 * NB * 32);
     // one workgroup per CU; the P workgroups of a column group are spread over the 8 XCDs, and the workgroups
     // that share A tiles (same position in different groups) sit on the same XCD

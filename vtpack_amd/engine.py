@@ -9,6 +9,7 @@ whole forward can be captured into a HIP graph.
 import torch
 
 from . import ops
+from .layers.dge import Deferred
 
 # The block has two independent chains before attention: the routing chain (router -> index->patch -> compress ->
 # q projection: small, latency-bound launches) and the key/value chain (LayerNorm of all tokens -> kv projection:
@@ -35,8 +36,24 @@ def _side_stream(device, slot=0):
     return s
 
 
+def prepare(model):
+    """Drop every derived copy of the model's weights (packed Linear weights, channels-last convolution weights) and
+    make the packed ones again now.  Derived copies are otherwise made on first use and refreshed whenever a weight's
+    storage, dtype, device or version counter changes; call this after writing weights in a way torch does not count
+    (`p.data.copy_(...)`, `p.data.mul_(...)`) and, optionally, before capturing a graph so that no packing kernel lands
+    in the capture."""
+    ops.invalidate_packed(model)
+    for mod in model.modules():
+        if hasattr(mod, "_vtdge_khwc"):
+            mod._vtdge_khwc = None
+        if isinstance(mod, torch.nn.Linear) and mod.weight.is_cuda and mod.weight.dtype == torch.bfloat16:
+            ops.packed_weight(mod.weight)
+    return model
+
+
 def _khwc_weight(conv):
-    """Conv2d weight [O, C, kh, kw] as a Linear weight over channels-last patches: [O, kh*kw*C]."""
+    """Conv2d weight [O, C, kh, kw] as a Linear weight over channels-last patches: [O, kh*kw*C] (see `prepare` for
+    when the cached copy is refreshed)."""
     w = conv.weight
     key = (w.data_ptr(), w._version, w.dtype, w.device)
     cached = getattr(conv, "_vtdge_khwc", None)
@@ -133,9 +150,21 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
     else:
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 
-    dge.states.update({"comp": comp, "input": x, "patches": patches, "batches": None, "batches_device": lengths,
-                       "offsets_device": offsets, "gate": gate, "size": (H, W), "num_extra_tokens": extra,
-                       "queries": q2})
+    # `states` as the reference's code reads it (vtpack/layers/dge.py:81-84): the host-side counts and the tensors cut
+    # to the live rows are produced on first read (one device->host copy, then cached); nothing is copied otherwise.
+    live = {}
+
+    def batches():
+        if "n" not in live:
+            live["n"] = lengths.cpu()
+        return live["n"]
+
+    def cut(t):
+        return lambda: t[:int(batches().sum())]
+
+    dge.states.update({"comp": Deferred(cut(comp)), "input": x, "patches": Deferred(cut(patches)),
+                       "batches": Deferred(batches), "batches_device": lengths, "offsets_device": offsets,
+                       "gate": gate, "size": (H, W), "num_extra_tokens": extra, "queries": Deferred(cut(q2))})
     if next_norm is not None:
         return out, out_ln          # out_ln is None when the fused kernel does not apply: the next block normalises
     return out
@@ -156,10 +185,13 @@ def model_forward(model, images):
     G = S // P
     C = model.embed_dim
     patches = images.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
-    x = torch.empty((B, 1 + G * G, C), dtype=images.dtype, device=images.device)
+    front = [t for t in (model.cls_token, getattr(model, "dist_token", None)) if t is not None]
+    extra = len(front)
+    x = torch.empty((B, extra + G * G, C), dtype=images.dtype, device=images.device)
     tok = ops.linear(patches, pe.proj.weight.reshape(C, Cin * P * P), pe.proj.bias)
-    x[:, 1:, :] = tok.view(B, G * G, C)
-    x[:, :1, :] = model.cls_token
+    x[:, extra:, :] = tok.view(B, G * G, C)
+    for e, t in enumerate(front):
+        x[:, e:e + 1, :] = t
     x += model.pos_embed
     x_ln = None
     blocks = list(model.blocks)
@@ -168,10 +200,22 @@ def model_forward(model, images):
             x, x_ln = block_forward(blk, x, G, G, x_ln=x_ln, next_norm=blocks[i + 1].norm1)
         else:
             x = block_forward(blk, x, G, G, x_ln=x_ln)
-    cls = ops.layernorm(x[:, 0, :], model.norm.weight, model.norm.bias, model.norm.eps)
-    if isinstance(model.head, torch.nn.Linear):
-        return ops.linear(cls, model.head.weight, model.head.bias)
-    return cls
+    nrm = model.norm
+
+    def head(lin, t):
+        return ops.linear(t, lin.weight, lin.bias) if isinstance(lin, torch.nn.Linear) else t
+
+    if extra == 0:      # no class token: the classifier sees the mean over all normalised tokens
+        return head(model.head, ops.layernorm(x, nrm.weight, nrm.bias, nrm.eps).mean(dim=1))
+    # only the rows of the extra tokens are needed after the last block
+    feats = ops.layernorm(x[:, :extra, :], nrm.weight, nrm.bias, nrm.eps)
+    if extra == 2:      # class + distillation token: the mean of the two classifiers (deit_dge.py:288-294)
+        return (head(model.head, feats[:, 0]) + head(model.head_dist, feats[:, 1])) / 2
+    cls = feats[:, 0]
+    pre = getattr(model, "pre_logits", None)
+    if isinstance(pre, torch.nn.Sequential):            # Linear + Tanh (deit_dge.py:198-204)
+        cls = torch.tanh(ops.linear(cls, pre.fc.weight, pre.fc.bias))
+    return head(model.head, cls)
 
 
 def pvt_forward(model, images):

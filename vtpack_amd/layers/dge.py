@@ -20,6 +20,40 @@ from .grained_sample import (grained_sample_compress, grained_sample_compress_de
                              grained_sample_decompress_dense, grained_sample_index_to_patch)
 
 
+class Deferred:
+    """A value of `states` that is only worked out when somebody reads it (see `States`)."""
+
+    def __init__(self, make):
+        self.make = make
+
+
+class States(dict):
+    """The `states` dict of a DynamicGrainedEncoder (vtpack/layers/dge.py:35-38, :81-84).
+
+    The fused inference path never copies the query counts to the host and works on buffers sized for the worst
+    case.  It therefore stores `batches` (CPU int64 lengths), `comp`, `patches` and `queries` as `Deferred` values:
+    reading one of them performs the device->host copy of the counts once and returns what the reference's code
+    expects, tensors cut to the live rows.  Code that never reads them never synchronises."""
+
+    def _resolve(self, key, value):
+        if isinstance(value, Deferred):
+            value = value.make()
+            dict.__setitem__(self, key, value)
+        return value
+
+    def __getitem__(self, key):
+        return self._resolve(key, dict.__getitem__(self, key))
+
+    def get(self, key, default=None):
+        return self._resolve(key, dict.get(self, key, default)) if key in self else default
+
+    def items(self):
+        return [(k, self[k]) for k in self.keys()]
+
+    def values(self):
+        return [self[k] for k in self.keys()]
+
+
 class DynamicRouter(nn.Module):
     """Region mean -> Linear(C, #splits).  vtpack/layers/dge.py:115-150."""
 
@@ -74,8 +108,8 @@ class DynamicGrainedEncoder(nn.Module):
         self.router = DynamicRouter(in_channels, split_sizes)
         self.complexity_handler = complexity_handler
         self.sparse_train = sparse_train
-        self.states = {"comp": None, "input": None, "patches": None, "batches": None, "gate": None, "size": None,
-                       "num_extra_tokens": 0}
+        self.states = States({"comp": None, "input": None, "patches": None, "batches": None, "gate": None,
+                              "size": None, "num_extra_tokens": 0})
 
     def get_complexity(self):
         # vtpack/layers/dge.py:40-59

@@ -14,6 +14,7 @@ Every block can run two ways at inference:
     device, see `vtpack_amd.engine.block_forward`.
 """
 import math
+from collections import OrderedDict
 from functools import partial
 
 import torch
@@ -117,29 +118,49 @@ class PatchEmbed(nn.Module):
 
 
 class VisionTransformer(nn.Module):
+    """vtpack/models/dge/deit_dge.py:133-299: class token, optional distillation token and second head
+    (`distilled`), optional pre-logits layer (`representation_size`, ignored with `distilled` as in the reference),
+    optional absence of the class token (`cls_token=False`: the head sees the mean over the tokens)."""
+
     def __init__(self, img_size=224, patch_size=16, in_chans=3, num_classes=1000, embed_dim=768, depth=12,
-                 num_heads=12, mlp_ratio=4., qkv_bias=True, qk_scale=None, norm_layer=None, split_sizes=(2, 1),
-                 fused=True):
+                 num_heads=12, mlp_ratio=4., qkv_bias=True, qk_scale=None, representation_size=None, distilled=False,
+                 drop_rate=0., attn_drop_rate=0., drop_path_rate=0., norm_layer=None, cls_token=True,
+                 split_sizes=(2, 1), fused=True):
         super().__init__()
+        # Dropout / stochastic depth are identities at inference; the rates are kept so that a training-mode forward
+        # can refuse them instead of silently training without the regularisers.
+        self.drop_rates = (drop_rate, attn_drop_rate, drop_path_rate)
         self.num_classes = num_classes
         self.num_features = self.embed_dim = embed_dim
-        self.num_tokens = 1
+        self.num_tokens = (1 if cls_token else 0) + (1 if distilled else 0)
         norm_layer = norm_layer or partial(nn.LayerNorm, eps=1e-6)
         self.patch_embed = PatchEmbed(img_size, patch_size, in_chans, embed_dim)
-        self.cls_token = nn.Parameter(torch.zeros(1, 1, embed_dim))
-        self.pos_embed = nn.Parameter(torch.zeros(1, self.patch_embed.num_patches + 1, embed_dim))
+        self.cls_token = nn.Parameter(torch.zeros(1, 1, embed_dim)) if cls_token else None
+        self.dist_token = nn.Parameter(torch.zeros(1, 1, embed_dim)) if distilled else None
+        self.pos_embed = nn.Parameter(torch.zeros(1, self.patch_embed.num_patches + self.num_tokens, embed_dim))
         self.blocks = nn.Sequential(*[
             Block(embed_dim, num_heads, mlp_ratio, qkv_bias, qk_scale, norm_layer, split_sizes, fused)
             for _ in range(depth)])
         self.norm = norm_layer(embed_dim)
-        self.head = nn.Linear(embed_dim, num_classes) if num_classes > 0 else nn.Identity()
+        if representation_size and not distilled:
+            self.num_features = representation_size
+            self.pre_logits = nn.Sequential(OrderedDict([("fc", nn.Linear(embed_dim, representation_size)),
+                                                         ("act", nn.Tanh())]))
+        else:
+            self.pre_logits = nn.Identity()
+        self.head = nn.Linear(self.num_features, num_classes) if num_classes > 0 else nn.Identity()
+        self.head_dist = None
+        if distilled:
+            self.head_dist = nn.Linear(embed_dim, num_classes) if num_classes > 0 else nn.Identity()
         self.fused = fused
         self._init_weights()
 
     def _init_weights(self):
         # timm's _init_vit_weights for the default scheme: trunc_normal(.02) weights, zero biases, unit LayerNorm
         nn.init.trunc_normal_(self.pos_embed, std=.02)
-        nn.init.trunc_normal_(self.cls_token, std=.02)
+        for tok in (self.cls_token, self.dist_token):
+            if tok is not None:
+                nn.init.trunc_normal_(tok, std=.02)
         for m in self.modules():
             if isinstance(m, nn.Linear):
                 nn.init.trunc_normal_(m.weight, std=.02)
@@ -158,6 +179,18 @@ class VisionTransformer(nn.Module):
             blk.fused = fused
         return self
 
+    def no_weight_decay(self):
+        return {"pos_embed", "cls_token"}
+
+    def get_classifier(self):
+        return self.head if self.dist_token is None else (self.head, self.head_dist)
+
+    def reset_classifier(self, num_classes, global_pool=""):
+        self.num_classes = num_classes
+        self.head = nn.Linear(self.embed_dim, num_classes) if num_classes > 0 else nn.Identity()
+        if self.num_tokens == 2:
+            self.head_dist = nn.Linear(self.embed_dim, num_classes) if num_classes > 0 else nn.Identity()
+
     def complexity(self, x):
         # deit_dge.py:234-249; call after a forward pass on x
         n = x.shape[1] * x.shape[2]
@@ -166,16 +199,35 @@ class VisionTransformer(nn.Module):
         return {"static": (sum(p["static"] for p in per) + base).mean(),
                 "dynamic": (sum(p["dynamic"] for p in per) + base).mean()}
 
-    def forward_features(self, x):
+    def embed_tokens(self, x):
+        """Patch tokens with the extra tokens in front (class, then distillation) plus the positions."""
         x = self.patch_embed(x)
-        x = torch.cat((self.cls_token.expand(x.shape[0], -1, -1), x), dim=1) + self.pos_embed
-        x = self.blocks(x)
-        return self.norm(x)[:, 0]
+        front = [t.expand(x.shape[0], -1, -1) for t in (self.cls_token, self.dist_token) if t is not None]
+        if self.cls_token is None and self.dist_token is not None:
+            raise ValueError("a distillation token needs a class token (deit_dge.py:270-275)")
+        return torch.cat(front + [x], dim=1) + self.pos_embed
+
+    def forward_features(self, x):
+        x = self.norm(self.blocks(self.embed_tokens(x)))
+        if self.cls_token is None:
+            return x
+        if self.dist_token is None:
+            return self.pre_logits(x[:, 0])
+        return x[:, 0], x[:, 1]
+
+    def classify(self, feats):
+        """deit_dge.py:286-299 on the output of forward_features."""
+        if self.head_dist is not None:
+            a, b = self.head(feats[0]), self.head_dist(feats[1])
+            return (a, b) if self.training else (a + b) / 2
+        return self.head(feats if self.cls_token is not None else feats.mean(dim=1))
 
     def forward(self, x):
         if self.fused and not self.training:
             return engine.model_forward(self, x)
-        return self.head(self.forward_features(x))
+        if self.training and any(self.drop_rates):
+            raise NotImplementedError("dropout / stochastic depth in training mode are not part of this package")
+        return self.classify(self.forward_features(x))
 
 
 def _deit_dge_s124(embed_dim, num_heads, **kwargs):

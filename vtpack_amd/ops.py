@@ -23,6 +23,31 @@ def _contig(t):
     return t if t.is_contiguous() else t.contiguous()
 
 
+def _check_like(x, **operands):
+    """Every given operand must have x's dtype and device: the kernels read all of them through one dtype code, so a
+    mismatch would make them read a buffer with the wrong element size (nn.Linear / nn.LayerNorm raise likewise)."""
+    for name, t in operands.items():
+        if t is None:
+            continue
+        if t.dtype != x.dtype:
+            raise TypeError(f"{name} is {t.dtype} but the activation is {x.dtype}: cast the module or the input")
+        if t.device != x.device:
+            raise TypeError(f"{name} is on {t.device} but the activation is on {x.device}")
+
+
+def _check_vector(name, t, n):
+    if t is not None and tuple(t.shape) != (n,):
+        raise ValueError(f"{name} has shape {tuple(t.shape)}, expected ({n},)")
+
+
+def _check_router(weight, bias, C, S, extra, H, W, region_size):
+    if tuple(weight.shape) != (S, C) or tuple(bias.shape) != (S,):
+        raise ValueError(f"router weight {tuple(weight.shape)} / bias {tuple(bias.shape)} do not map {C} channels")
+    if extra < 0 or H % region_size or W % region_size:
+        raise ValueError(f"a {H}x{W} token grid with {extra} extra tokens does not tile into regions of "
+                         f"{region_size}")
+
+
 def router(x, weight, bias, H, W, region_size, want_gate=True):
     """AvgPool(R) -> Linear -> argmax on the spatial tokens of x [B, extra+H*W, C].
 
@@ -33,6 +58,7 @@ def router(x, weight, bias, H, W, region_size, want_gate=True):
     B, N, C = x.shape
     S = weight.shape[0]
     extra = N - H * W
+    _check_router(weight, bias, C, S, extra, H, W, region_size)
     Hr, Wr = H // region_size, W // region_size
     gate = torch.empty((B, Hr, Wr, S), dtype=x.dtype, device=x.device) if want_gate else None
     indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
@@ -56,6 +82,7 @@ def router_layernorm(x, weight, bias, H, W, region_size, ln_weight, ln_bias, ln_
     B, N, C = x.shape
     S = weight.shape[0]
     extra = N - H * W
+    _check_router(weight, bias, C, S, extra, H, W, region_size)
     Hr, Wr = H // region_size, W // region_size
     gate = torch.empty((B, Hr, Wr, S), dtype=x.dtype, device=x.device) if want_gate else None
     indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
@@ -70,6 +97,8 @@ def router_layernorm(x, weight, bias, H, W, region_size, ln_weight, ln_bias, ln_
 def index_to_patch(indices, splits, region_size, num_extra_tokens, capacity=None):
     """Device-only compaction: (patches [capacity,4], offsets [B+1], lengths [B]), all on the GPU."""
     _need_gpu(indices, splits)
+    if indices.dtype != torch.int64 or splits.dtype != torch.int64 or indices.dim() != 3:
+        raise TypeError("indices must be int64 [B, Hr, Wr] and splits int64")
     indices, splits = _contig(indices), _contig(splits)
     B, Hr, Wr = indices.shape
     if capacity is None:
@@ -85,9 +114,15 @@ def index_to_patch(indices, splits, region_size, num_extra_tokens, capacity=None
 def compress(x, patches, width, num_extra_tokens, rows_dev=None, rows=None, ln_weight=None, ln_bias=None,
              ln_eps=1e-6):
     """x [B,N,C] -> comp [rows,C] (and LayerNorm(comp) when ln_weight is given)."""
-    _need_gpu(x, patches)
+    _need_gpu(x, patches, ln_weight, ln_bias)
     x, patches = _contig(x), _contig(patches)
     B, N, C = x.shape
+    _check_like(x, ln_weight=ln_weight, ln_bias=ln_bias)
+    _check_vector("ln_weight", ln_weight, C)
+    _check_vector("ln_bias", ln_bias, C)
+    if (ln_weight is None) != (ln_bias is None):
+        raise ValueError("the fused LayerNorm needs both its weight and its bias")
+    ln_weight, ln_bias = (None, None) if ln_weight is None else (_contig(ln_weight), _contig(ln_bias))
     rows = patches.shape[0] if rows is None else rows
     out = torch.empty((rows, C), dtype=x.dtype, device=x.device)
     ln_out = torch.empty_like(out) if ln_weight is not None else None
@@ -104,6 +139,10 @@ def decompress(inp, patches, reference, width, num_extra_tokens, add_ref=True, s
     inp, patches, reference = _contig(inp), _contig(patches), _contig(reference)
     sub = None if sub is None else _contig(sub)
     B, N, C = reference.shape
+    _check_like(inp, reference=reference, sub=sub, out=out)
+    if inp.shape[-1] != C or (sub is not None and sub.shape != inp.shape):
+        raise ValueError(f"packed rows {tuple(inp.shape)} / {None if sub is None else tuple(sub.shape)} do not match "
+                         f"the reference's {C} channels")
     rows = patches.shape[0] if rows is None else rows
     if out is None:
         out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
@@ -120,6 +159,12 @@ def decompress_layernorm(inp, patches, reference, width, num_extra_tokens, ln_we
     inp, patches, reference = _contig(inp), _contig(patches), _contig(reference)
     sub = None if sub is None else _contig(sub)
     B, N, C = reference.shape
+    _check_like(inp, reference=reference, sub=sub, ln_weight=ln_weight, ln_bias=ln_bias)
+    _check_vector("ln_weight", ln_weight, C)
+    _check_vector("ln_bias", ln_bias, C)
+    if inp.shape[-1] != C or (sub is not None and sub.shape != inp.shape):
+        raise ValueError("packed rows do not match the reference's channel count")
+    ln_weight, ln_bias = _contig(ln_weight), _contig(ln_bias)
     rows = patches.shape[0] if rows is None else rows
     out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
     ln_out = torch.empty_like(out)
@@ -138,21 +183,48 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     _need_gpu(x, weight, bias)
     x = _contig(x)
     C = x.shape[-1]
+    _check_like(x, weight=weight, bias=bias, out=out)
+    _check_vector("weight", weight, C)
+    _check_vector("bias", bias, C)
+    weight, bias = _contig(weight), _contig(bias)
     rows = x.numel() // C
     if out is None:
         out = torch.empty_like(x)
+    elif out.shape != x.shape or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor of the input's shape")
     call("vtdge_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(rows_dev), rows, C, float(eps),
          dtype_code(x), stream_ptr(), tag=("layernorm", rows_dev is not None, rows, C))
     return out
 
 
 PACK_WEIGHTS = True     # module switch (tests compare the two paths)
+_pack_epoch = 0         # bumped by invalidate_packed(): every packed copy made before is stale
+
+
+def invalidate_packed(obj=None):
+    """Forget packed copies of Linear weights: all of them (no argument), one tensor's, or those of every parameter
+    of a module.
+
+    The copy is keyed on the weight's storage address, shape, dtype, device and version counter, which covers
+    `load_state_dict`, `.to()` / `.bfloat16()`, optimiser steps and every in-place torch op on the parameter.  It does
+    NOT see writes that bypass the version counter: `w.data.copy_(...)`, `w.data.mul_(...)`, a raw kernel writing
+    into the storage.  After such a write call this function (or `engine.prepare(model)`) before the next forward;
+    otherwise the weight-stationary kernels keep multiplying by the old weights."""
+    global _pack_epoch
+    if obj is None:
+        _pack_epoch += 1
+        return
+    tensors = obj.parameters() if isinstance(obj, torch.nn.Module) else [obj]
+    for t in tensors:
+        if getattr(t, "_vtdge_packed", None) is not None:
+            t._vtdge_packed = None
 
 
 def packed_weight(weight):
     """The copy of a Linear weight [N, K] in the register order of the weight-stationary kernels, made once per
-    weight tensor and version and kept on the tensor object; None when the kernels for this shape take W as it is."""
-    key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, weight.device)
+    weight tensor and version and kept on the tensor object; None when the kernels for this shape take W as it is.
+    See `invalidate_packed` for the one kind of edit the key cannot detect."""
+    key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, weight.device, _pack_epoch)
     cached = getattr(weight, "_vtdge_packed", None)
     if cached is not None and cached[0] == key:
         return cached[1]
@@ -176,18 +248,27 @@ def packed_weight(weight):
 def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=None):
     """out = act(a @ weight.T + bias) + residual; a [..., K] (last dim contiguous), weight [N, K]."""
     _need_gpu(a, weight, bias, residual)
+    _check_like(a, weight=weight, bias=bias, residual=residual, out=out)
     K = a.shape[-1]
+    if weight.dim() != 2 or weight.shape[1] != K:
+        raise ValueError(f"weight {tuple(weight.shape)} does not take inputs of width {K}")
     a2 = a.reshape(-1, K)
     if a2.stride(-1) != 1:
         a2 = a2.contiguous()
     weight = _contig(weight)
     N = weight.shape[0]
+    _check_vector("bias", bias, N)
+    bias = None if bias is None else _contig(bias)
     rows = a2.shape[0]
     if out is None:
         out = torch.empty(a.shape[:-1] + (N,), dtype=a.dtype, device=a.device)
+    elif out.numel() != rows * N or out.shape[-1] != N:
+        raise ValueError(f"out {tuple(out.shape)} does not hold {rows} rows of {N}")
     o2 = out.view(-1, N)
     r2 = None
     if residual is not None:
+        if residual.numel() != rows * N or residual.shape[-1] != N:
+            raise ValueError(f"residual {tuple(residual.shape)} does not hold {rows} rows of {N}")
         r2 = residual.reshape(-1, N)
         if r2.stride(-1) != 1:
             r2 = r2.contiguous()
@@ -203,11 +284,16 @@ def sparse_attention(q, k, v, offsets, scale, num_heads, max_rows_per_sample, ou
     """Strided form.  q [L, h*d]; k, v [B, n, h*d]-like views (last dim contiguous, any batch/token strides);
     offsets int64 [B+1] on the device.  Returns [L, h*d] with channel = head*d + j."""
     _need_gpu(q, k, v, offsets)
+    _check_like(q, k=k, v=v, out=out)
     L, C = q.shape
     d = C // num_heads
     B, n = k.shape[0], k.shape[1]
-    assert k.stride(-1) == 1 and v.stride(-1) == 1 and q.stride(-1) == 1
-    assert k.stride() == v.stride()
+    if k.shape != v.shape or k.shape[-1] != C or C % num_heads:
+        raise ValueError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not share {num_heads} heads")
+    if offsets.dtype != torch.int64 or offsets.numel() != B + 1:
+        raise ValueError("offsets must be int64 [B + 1]")
+    if not (k.stride(-1) == 1 and v.stride(-1) == 1 and q.stride(-1) == 1 and k.stride() == v.stride()):
+        raise ValueError("q, k and v need a contiguous last dimension, k and v the same strides")
     if out is None:
         out = torch.empty((L, C), dtype=q.dtype, device=q.device)
     call("vtdge_sparse_attention", ptr(q), q.stride(0), d, ptr(k), ptr(v), k.stride(0), k.stride(1), d,
