@@ -128,7 +128,7 @@ def _assert_bf16_gates_differ_only_at_near_ties(model, traces, floor):
     print(f"bf16 gate agreement {same}/{total}, largest margin among disagreements {worst:.4f}, "
           f"largest |logit| {scale:.2f}")
     assert same / total >= floor
-    assert worst <= 8 * 2.0 ** -8 * max(scale, 1.0), (worst, scale)
+    assert worst <= 4 * 2.0 ** -8 * max(scale, 1.0), (worst, scale)
 
 
 @pytest.mark.parametrize("fused", [True, False])
@@ -261,7 +261,7 @@ def test_deit_variants_fp32(dev, variant, fused):
     set_synthetic_router(m, 5)
     with torch.no_grad():
         for name, p in m.named_parameters():
-            if p.dim() == 1 and "router" not in name:
+            if p.dim() == 1 and p.is_floating_point() and "router" not in name:
                 p.add_(0.1 * torch.randn_like(p))
     m = m.eval().to(dev)
     img = synthetic_images(3, 128, seed=8)
