@@ -388,15 +388,16 @@ def cpu_baseline(args, torch, model, images, heads):
         run = lambda: torch_ref.pvt_dge_forward(sd, img, heads, model.depths, sr)  # noqa: E731
     with torch.no_grad():
         run()
+        run()
         times = []
-        for _ in range(3):
+        for _ in range(5):
             t0 = time.perf_counter()
             run()
             times.append(time.perf_counter() - t0)
-    med = sorted(times)[1]
+    med = sorted(times)[2]
     return {"value": round(sample / med, 2), "unit": "images/s", "cores": threads, "kind": "port",
             "sample": f"{sample} images of the same workload, fp32 torch-CPU restatement (oracle/torch_ref.py), "
-                      f"median of 3 after 1 warm-up, {threads} threads"}
+                      f"median of 5 after 2 warm-ups, {threads} threads"}
 
 
 def main():
@@ -407,7 +408,7 @@ def main():
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size")
     ap.add_argument("--no-graph", action="store_true", help="time the eager path instead of a HIP graph replay")
-    ap.add_argument("--cpu-sample", type=int, default=32, help="images in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=128, help="images in the CPU baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (the path shards along the batch with no exchange step)."

@@ -133,3 +133,75 @@ def test_dense_training_branch_equals_the_sparse_statement_on_cpu():
     out.square().sum().backward()
     assert x.grad is not None and float(x.grad.abs().max()) > 0
     assert float(d.router.gate.weight.grad.abs().max()) > 0
+
+
+def test_checkpoint_round_trip(tmp_path):
+    """A checkpoint written the way the reference's training loop writes it ({"model": state_dict, ...}) loads
+    through a loader that executes nothing from the file, into the same keys and values (main.py:372-379)."""
+    from vtpack_amd import harness
+    from vtpack_amd.models.dge import deit_dge_s124_tiny_patch16_256
+    torch.manual_seed(0)
+    a = deit_dge_s124_tiny_patch16_256(num_classes=10)
+    with torch.no_grad():
+        for p in a.parameters():
+            if p.is_floating_point():
+                p.add_(0.01 * torch.randn_like(p))
+    path = tmp_path / "checkpoint.pth"
+    torch.save({"model": a.state_dict(), "epoch": 7, "args": {"dge_budget": 0.5}}, path)
+    torch.manual_seed(1)
+    b = deit_dge_s124_tiny_patch16_256(num_classes=10)
+    rest = harness.load_checkpoint(b, path)
+    assert rest == {"epoch": 7, "args": {"dge_budget": 0.5}}
+    sa, sb = a.state_dict(), b.state_dict()
+    assert list(sa) == list(sb) and all(torch.equal(sa[k], sb[k]) for k in sa)
+    assert sb["blocks.0.dge.splits"].dtype == torch.int64
+    # a bare state dict and a DistributedDataParallel-style wrapper are accepted as well
+    torch.save(a.state_dict(), path)
+
+    class Wrapped(torch.nn.Module):
+        def __init__(self, m):
+            super().__init__()
+            self.module = m
+
+    torch.manual_seed(2)
+    c = Wrapped(deit_dge_s124_tiny_patch16_256(num_classes=10))
+    assert harness.load_checkpoint(c, path) == {}
+    assert all(torch.equal(sa[k], v) for k, v in c.module.state_dict().items())
+    # a checkpoint of another architecture is refused, not half-loaded
+    with pytest.raises(RuntimeError):
+        harness.load_checkpoint(deit_dge_s124_tiny_patch16_256(num_classes=10, distilled=True), path)
+
+
+def test_evaluate_meters_on_a_plain_model():
+    """The evaluation loop's meters (vtpack/engine/engine.py:102-147): per-batch means of the loss, accuracies
+    weighted by the batch size, against a direct computation."""
+    from vtpack_amd import harness
+    torch.manual_seed(0)
+    net = torch.nn.Sequential(torch.nn.Flatten(), torch.nn.Linear(3 * 8 * 8, 7))
+    batches = [(torch.randn(5, 3, 8, 8), torch.randint(0, 7, (5,))), (torch.randn(3, 3, 8, 8), torch.randint(0, 7, (3,)))]
+    stats = harness.evaluate(batches, net, "cpu")
+    assert set(stats) == {"loss", "acc1", "acc5"}
+    with torch.no_grad():
+        outs = [net(x) for x, _ in batches]
+    losses = [float(torch.nn.functional.cross_entropy(o, t)) for o, (_, t) in zip(outs, batches)]
+    assert stats["loss"] == pytest.approx(sum(losses) / 2)
+    hits1 = sum(int((o.argmax(1) == t).sum()) for o, (_, t) in zip(outs, batches))
+    hits5 = sum(int((o.topk(5, 1).indices == t[:, None]).any(1).sum()) for o, (_, t) in zip(outs, batches))
+    assert stats["acc1"] == pytest.approx(100.0 * hits1 / 8) and stats["acc5"] == pytest.approx(100.0 * hits5 / 8)
+
+
+def test_budget_loss_from_planted_gates():
+    """loss_dge = scale * (dynamic / static - budget)^2 (vtpack/engine/engine.py:58-63) on the counter's output."""
+    from vtpack_amd import harness
+    from vtpack_amd.models.dge import deit_dge_s124_tiny_patch16_256
+    m = deit_dge_s124_tiny_patch16_256().eval()
+    img = torch.zeros(2, 3, 256, 256)
+    _fake_states(m, 2)
+    loss, ratio, comp = harness.budget_loss(m, img, dge_budget=0.5, dge_lr_scale=3.0)
+    assert float(ratio) == pytest.approx(float(comp["dynamic"]) / float(comp["static"]))
+    assert float(loss) == pytest.approx(3.0 * (float(ratio) - 0.5) ** 2)
+    _fake_states(m, 0)
+    loss, ratio, _ = harness.budget_loss(m, img, dge_budget=1.0)
+    assert float(ratio) == pytest.approx(1.0) and float(loss) == pytest.approx(0.0, abs=1e-12)
+    # the per-encoder ratio of engine.py:20-32 on the same states
+    assert float(harness.get_complexity(m)) == pytest.approx(1.0)
