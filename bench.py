@@ -91,7 +91,9 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
     if name == "vtdge_sparse_attention":
         if dt == "bf16" and tag[3] == 64:
-            return "sparse_attention_bf16_d64_resident_kernel" if tag[4] <= 288 else "sparse_attention_bf16_d64_kernel"
+            if tag[4] <= 288:
+                return f"sparse_attention_bf16_d64_pipelined_kernel<{-(-tag[4] // 32)}>"
+            return "sparse_attention_bf16_d64_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
         return f"router_kernel<{T}, 4, {gs(tag[1])}, false>"     # region size 4 in every model of these workloads

@@ -1,14 +1,13 @@
 // Sparse attention, bf16 / head_dim 64 fast path (gfx950).
 //
-// Same mathematics and MFMA mapping as attention.hip (S^T = K Q^T, O^T = V^T P^T, online softmax, a lane owns one
-// query), restructured around what limits this operator at head_dim 64: the softmax VALU work (about 8 lane-ops
-// per score against 0.25 MFMA cycles) and the K/V staging.
-//   * K/V stages of 128 keys are double buffered in LDS: while stage s is multiplied, K of stage s+1 arrives by
-//     direct loads (global_load_lds, 128-byte rows, XOR-swizzled 16-byte chunks, no padding) and V of stage s+1
-//     sits in registers, to be written transposed ([d][key], key groups XOR-swizzled by d to spread the 2-byte
-//     writes over the banks) after the multiply.  One barrier per stage.
-//   * the softmax works in the log2 domain: p = exp2(fma(s, scale*log2(e), -m)); the running maximum is taken on
-//     the raw scores (scale > 0), and key masking is only applied in a stage that contains the end of the keys.
+// Same mathematics and MFMA mapping as attention.hip (S^T = K Q^T, O^T = V^T P^T, a lane owns one query),
+// restructured around what limits this operator at head_dim 64: the softmax's vector instructions (a wave issues
+// one every ~5 clocks, and there are about five per score against a quarter of an MFMA clock) and the K/V staging.
+//   * up to 288 keys (the 256 px models): K and V of a (sample, head) stay resident in LDS, double buffered across
+//     items by direct loads; V is transposed by the LDS read itself (ds_read_b64_tr_b16); the tile loop is a
+//     hand-ordered software pipeline in which the reference of the softmax rides in the MFMA accumulator;
+//   * longer sequences (512 px, spatially reduced PVT stages): K/V stages of 128 keys double buffered in LDS, K by
+//     direct loads, V through registers and transposed writes, online softmax in the log2 domain.
 #include "common.h"
 #include <stdlib.h>
 
@@ -114,20 +113,8 @@ __device__ __forceinline__ void attn_store(bf16_t *op, const f32x16 (&o)[2], flo
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Resident variant for short key sequences (n <= 288, e.g. 257 tokens at 256 px): one workgroup per (sample,
-// head) stages that sample's whole K and V^T once (one exposed memory latency, no re-staging per query chunk),
-// then its four waves walk the sample's 32-row query tiles independently, without further barriers.
-//
-// V^T layout in LDS: row d holds the keys in groups of 16; inside a group key 8h + 4g + j sits at position
-// 8g + 4h + j, so the 8 keys a lane feeds to one MFMA (its P fragment holds keys 4g + j and 8 + 4g + j) are 16
-// contiguous bytes; the group index is XOR-ed with (d >> 4) & 3, which spreads the 2-byte transposing writes over
-// all banks; rows are padded by 16 B, which keeps the 16-byte fragment reads conflict free.
-//
-// Softmax: the keys are cut into equal stages of at most 4 blocks of 32 (257 keys: 3 stages of 3 blocks).  The
-// running reference m of a row is only raised when a stage's maximum exceeds it by more than 8 (log2 units), so
-// p = exp2(s*c - m) <= 256 and the rescaling of the output accumulators is skipped in most stages; the result is
-// the same softmax (any reference cancels in the final division).
-constexpr float ATT_RESCALE = 8.0f;
+constexpr float ATT_RESCALE = 8.0f;   // log2 units a score may exceed its row's reference by before that is raised
+constexpr int ATT_TBL = 512;          // items per workgroup whose first row and query count are kept in LDS
 
 // acc + lo + hi of a packed bf16 pair in fp32 (v_dot2c_f32_bf16 against (1, 1))
 __device__ __forceinline__ float bf16_pair_sum(uint32_t pair, float acc)
@@ -136,200 +123,388 @@ __device__ __forceinline__ float bf16_pair_sum(uint32_t pair, float acc)
                                            acc, false);
 }
 
-template <int NB, bool FULL>
-__device__ __forceinline__ void attn_stage_resident(const unsigned char *kp, const unsigned char *vrow0,
-                                                    const unsigned char *vrow1, int vsw0, int vsw1, int key0, int n,
-                                                    int lg, const int (&cs)[4], const u32x4 (&qf)[4], f32x16 (&o)[2],
-                                                    float &m_used, float &l_run, float c)
+// ---------------------------------------------------------------------------------------------------------
+// One 32-query tile against all resident keys, software-pipelined over blocks of 32 keys: while the vector ALU
+// turns the scores of block kb into probabilities, the matrix pipe already multiplies K of block kb+1 with Q, and
+// every fragment of K is read from LDS one block before the MFMA that consumes it.  The order of the instructions
+// below is the order they are meant to issue in (pinned by scheduling barriers): a wave issues one vector
+// instruction every ~5 clocks (v_exp_f32 ~12, v_cvt_pk_bf16_f32 ~8) and the softmax is what the tile waits for, so
+// its instruction count is what is kept small; the MFMAs ride along.
+//
+// The queries are multiplied by scale * log2(e) when they are loaded, and the score MFMAs start from an
+// accumulator that holds minus the row's reference m: a block's scores come out of the matrix pipe as
+// s' = log2-scaled score - m, and a probability is one v_exp_f32 of that.  The reference of a row is its maximum
+// over the first block; later it is only raised (and the running sums rescaled) when some score of a block exceeds
+// it by more than ATT_RESCALE, which is decided before the next block's MFMAs are issued.  Any reference cancels in
+// the final division, so this is the same softmax as the max-subtracted one.
+struct AttnTile {
+    const unsigned char *krow;      // K row `lr` of block 0 in LDS
+    const unsigned char *vlane;     // this lane's source address for the transposing reads of V, block 0, d < 32
+    int n, lg;
+};
+
+__device__ __forceinline__ u32x4 att_read_k(const AttnTile &t, const int (&cs)[4], int kb, int sl)
 {
-    // byte offsets of this stage's 16-key groups in the two V^T rows of the lane
-    int voff0[2 * NB], voff1[2 * NB];
+    return *reinterpret_cast<const u32x4 *>(t.krow + kb * 32 * 128 + cs[sl]);
+}
+// V stays row-major in LDS ([key][d], 128-byte rows like K) and is transposed on the way to the registers:
+// ds_read_b64_tr_b16 works on blocks of 16 lanes; source lane 4e + r of a block names four consecutive 16-bit
+// elements, and lane i of the block receives, as its element e, column (i & 3) of source lane 4e + (i >> 2).  With
+// source lane 4e + r pointing at key k0 + e, channels d0 + 4r .. d0 + 4r + 3, lane i receives keys k0 .. k0 + 3 of
+// channel d0 + i: four K-elements of a row of V^T.  The first operand of O^T += V^T P^T wants, in lane (lr, lg),
+// channel 32 db + lr and the eight keys the lane's own P fragment holds (16 h + 4 lg + j and 16 h + 8 + 4 lg + j,
+// j < 4): two such reads, with k0 = 16 h + 4 lg (+ 8) and d0 = 32 db + 16 (block & 1).  Rows are stored with their
+// 16-byte chunks XOR-ed by 2 (key & 3), so the sixteen 8-byte pieces of a block come from sixteen different bank
+// groups; the XOR constant of a lane does not depend on kb, h or the +8, and db = 1 is the address XOR 64.
+typedef short att_v4s __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 att_tr_read(const unsigned char *p)
+{
+    const att_v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) att_v4s *)(uint32_t)(uintptr_t)p);
+    return __builtin_bit_cast(u32x2, r);
+}
+__device__ __forceinline__ const unsigned char *att_v_lane(const unsigned char *vbase, int lane)
+{
+    const int blk = lane >> 4, i = lane & 15;
+    const int e = i >> 2, r = i & 3;                   // role of this lane as a source
+    const int key = 4 * (blk >> 1) + e;                 // + 32 kb + 16 h (+ 8)
+    const int chunk = (2 * (blk & 1) + (r >> 1)) ^ (2 * (key & 3));
+    return vbase + key * 128 + chunk * 16 + 8 * (r & 1);
+}
+__device__ __forceinline__ void att_read_v(const AttnTile &t, int kb, u32x4 (&vf)[4])
+{
 #pragma unroll
-    for (int g = 0; g < 2 * NB; g++) {
-        voff0[g] = ((key0 + 16 * g) ^ vsw0) * 2;
-        voff1[g] = ((key0 + 16 * g) ^ vsw1) * 2;
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int db = 0; db < 2; db++) {
+            const unsigned char *p =
+                reinterpret_cast<const unsigned char *>((uintptr_t)(t.vlane + (kb * 32 + 16 * h) * 128) ^ (64u * db));
+            const u32x2 lo = att_tr_read(p), hi = att_tr_read(p + 8 * 128);
+            vf[2 * h + db].x = lo.x;
+            vf[2 * h + db].y = lo.y;
+            vf[2 * h + db].z = hi.x;
+            vf[2 * h + db].w = hi.y;
+        }
+}
+#define VT_PIN() __builtin_amdgcn_sched_barrier(0)
+__device__ __forceinline__ f32x16 att_mfma(const u32x4 &a, const u32x4 &b, const f32x16 &acc)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
+                                                   0, 0);
+}
+// q * f for the packed bf16 pairs of a fragment (round to nearest even)
+__device__ __forceinline__ u32x4 att_scale_frag(const u32x4 &q, float f)
+{
+    u32x4 r;
+    r.x = pack_bf16x2(bf16lo(q.x) * f, bf16hi(q.x) * f);
+    r.y = pack_bf16x2(bf16lo(q.y) * f, bf16hi(q.y) * f);
+    r.z = pack_bf16x2(bf16lo(q.z) * f, bf16hi(q.z) * f);
+    r.w = pack_bf16x2(bf16lo(q.w) * f, bf16hi(q.w) * f);
+    return r;
+}
+__device__ __forceinline__ float att_max16(const f32x16 &s)
+{
+    const float a = fmaxf(fmaxf(fmaxf(s[0], s[1]), s[2]), fmaxf(fmaxf(s[3], s[4]), s[5]));
+    const float b = fmaxf(fmaxf(fmaxf(s[6], s[7]), s[8]), fmaxf(fmaxf(s[9], s[10]), s[11]));
+    return fmaxf(fmaxf(a, b), fmaxf(fmaxf(fmaxf(s[12], s[13]), s[14]), s[15]));
+}
+
+// One step of the pipeline: softmax of block kb (scores relative to the reference in `sc`) and O^T += V^T P^T,
+// interleaved with the score MFMAs of block kb+1 (fragments in `kf` -> `sn`, when NEXT); each fragment of K is
+// replaced by that of block kb+2 (when NEXT2) as soon as its MFMA has been issued.  MASK: block kb is the last
+// one and runs past the keys.
+template <bool NEXT, bool NEXT2, bool MASK>
+__device__ __forceinline__ void att_step(const AttnTile &t, const int (&cs)[4], int kb, f32x16 &sc, f32x16 &sn,
+                                         u32x4 (&kf)[4], const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm,
+                                         float (&l)[2])
+{
+    u32x4 vf[4];
+    att_read_v(t, kb, vf);
+    if constexpr (MASK) {
+        const int lim = t.n - kb * 32 - 4 * t.lg;
+#pragma unroll
+        for (int e = 0; e < 16; e++)
+            if (8 * (e >> 2) + (e & 3) >= lim) sc[e] = -INFINITY;
     }
-    f32x16 s[NB];
-    float mx = -INFINITY;
+    const float mx = att_max16(sc);
+    if (__builtin_amdgcn_ballot_w64(mx > ATT_RESCALE) != 0) {      // wave-uniform and rare
+        const float mrow = fmaxf(mx, __shfl_xor(mx, 32, WAVE));     // both lanes of a row decide alike
+        const float delta = mrow > ATT_RESCALE ? mrow : 0.f;
+        const float alpha = __builtin_amdgcn_exp2f(-delta);
+        l[0] *= alpha;
+        l[1] *= alpha;
 #pragma unroll
-    for (int kb = 0; kb < NB; kb++) {
-#pragma unroll
-        for (int e = 0; e < 16; e++) s[kb][e] = 0.f;
-#pragma unroll
-        for (int sl = 0; sl < 4; sl++) {
-            const u32x4 kf = *reinterpret_cast<const u32x4 *>(kp + kb * 32 * 128 + cs[sl]);
-            Slab<bf16_t>::mma(kf, qf[sl], s[kb]);
+        for (int e = 0; e < 16; e++) {
+            o[0][e] *= alpha;
+            o[1][e] *= alpha;
+            sc[e] -= delta;
+            negm[e] -= delta;
         }
-        if constexpr (!FULL) {
-            if (kb == NB - 1) {        // only the last block of the last stage can run past the keys
-                const int lim = n - key0 - kb * 32 - 4 * lg;
-#pragma unroll
-                for (int e = 0; e < 16; e++)
-                    if (8 * (e >> 2) + (e & 3) >= lim) s[kb][e] = -INFINITY;
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 16; e++) mx = fmaxf(mx, s[kb][e]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * c;
-    if (__builtin_amdgcn_ballot_w64(mx > m_used + ATT_RESCALE) != 0) {      // wave-uniform; rare after stage 0
-        const float m_new = mx > m_used + ATT_RESCALE ? mx : m_used;
-        const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);           // 0 on the first stage (m_used = -inf)
-        l_run *= alpha;
-        if (__builtin_amdgcn_ballot_w64(m_used > -INFINITY) != 0) {          // nothing accumulated yet on stage 0
+    VT_PIN();
+    u32x4 pf[2];
+    float p[16];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+    for (int e = 0; e < 4; e++) p[e] = __builtin_amdgcn_exp2f(sc[e]);
+    VT_PIN();
+    if constexpr (NEXT) sn = att_mfma(kf[0], qf[0], negm);
+    if constexpr (NEXT2) kf[0] = att_read_k(t, cs, kb + 2, 0);
+    VT_PIN();
 #pragma unroll
-                for (int e = 0; e < 16; e++) o[i][e] *= alpha;
-        }
-        m_used = m_new;
+    for (int e = 4; e < 8; e++) p[e] = __builtin_amdgcn_exp2f(sc[e]);
+    VT_PIN();
+    if constexpr (NEXT) sn = att_mfma(kf[1], qf[1], sn);
+    if constexpr (NEXT2) kf[1] = att_read_k(t, cs, kb + 2, 1);
+    VT_PIN();
+    pf[0].x = pack_bf16x2(p[0], p[1]);
+    pf[0].y = pack_bf16x2(p[2], p[3]);
+    pf[0].z = pack_bf16x2(p[4], p[5]);
+    pf[0].w = pack_bf16x2(p[6], p[7]);
+    // the row sum is taken over the rounded probabilities, the values the second MFMA multiplies with
+    l[0] = bf16_pair_sum(pf[0].x, l[0]);
+    l[1] = bf16_pair_sum(pf[0].y, l[1]);
+    l[0] = bf16_pair_sum(pf[0].z, l[0]);
+    l[1] = bf16_pair_sum(pf[0].w, l[1]);
+    VT_PIN();
+    o[0] = att_mfma(vf[0], pf[0], o[0]);
+    VT_PIN();
+#pragma unroll
+    for (int e = 8; e < 12; e++) p[e] = __builtin_amdgcn_exp2f(sc[e]);
+    VT_PIN();
+    o[1] = att_mfma(vf[1], pf[0], o[1]);
+    VT_PIN();
+#pragma unroll
+    for (int e = 12; e < 16; e++) p[e] = __builtin_amdgcn_exp2f(sc[e]);
+    VT_PIN();
+    if constexpr (NEXT) sn = att_mfma(kf[2], qf[2], sn);
+    if constexpr (NEXT2) kf[2] = att_read_k(t, cs, kb + 2, 2);
+    VT_PIN();
+    pf[1].x = pack_bf16x2(p[8], p[9]);
+    pf[1].y = pack_bf16x2(p[10], p[11]);
+    pf[1].z = pack_bf16x2(p[12], p[13]);
+    pf[1].w = pack_bf16x2(p[14], p[15]);
+    VT_PIN();
+    if constexpr (NEXT) sn = att_mfma(kf[3], qf[3], sn);
+    if constexpr (NEXT2) kf[3] = att_read_k(t, cs, kb + 2, 3);
+    VT_PIN();
+    l[0] = bf16_pair_sum(pf[1].x, l[0]);
+    l[1] = bf16_pair_sum(pf[1].y, l[1]);
+    l[0] = bf16_pair_sum(pf[1].z, l[0]);
+    l[1] = bf16_pair_sum(pf[1].w, l[1]);
+    VT_PIN();
+    o[0] = att_mfma(vf[2], pf[1], o[0]);
+    o[1] = att_mfma(vf[3], pf[1], o[1]);
+    VT_PIN();
+}
+
+// Block 0 of a tile: raw scores, the row's first reference, and the accumulator the later score MFMAs start from.
+__device__ __forceinline__ void att_first_block(const AttnTile &t, const int (&cs)[4], int nblk, u32x4 (&kf)[4],
+                                                const u32x4 (&qf)[4], f32x16 &s0, f32x16 &negm)
+{
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) kf[sl] = att_read_k(t, cs, 0, sl);
+    s0 = att_mfma(kf[0], qf[0], zero);
+    s0 = att_mfma(kf[1], qf[1], s0);
+    s0 = att_mfma(kf[2], qf[2], s0);
+    s0 = att_mfma(kf[3], qf[3], s0);
+    if (nblk > 1) {
+#pragma unroll
+        for (int sl = 0; sl < 4; sl++) kf[sl] = att_read_k(t, cs, 1, sl);
     }
+    if (nblk == 1 && (t.n & 31) != 0) {        // a lone, partial block: its missing keys must not set the reference
+        const int lim = t.n - 4 * t.lg;
 #pragma unroll
-    for (int kb = 0; kb < NB; kb++) {
+        for (int e = 0; e < 16; e++)
+            if (8 * (e >> 2) + (e & 3) >= lim) s0[e] = -INFINITY;
+    }
+    float m = att_max16(s0);
+    m = fmaxf(m, __shfl_xor(m, 32, WAVE));         // key 0 always exists: m is finite
 #pragma unroll
-        for (int e = 0; e < 16; e++) s[kb][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], c, -m_used));
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            u32x4 pf;
-            pf.x = pack_bf16x2(s[kb][8 * t + 0], s[kb][8 * t + 1]);
-            pf.y = pack_bf16x2(s[kb][8 * t + 2], s[kb][8 * t + 3]);
-            pf.z = pack_bf16x2(s[kb][8 * t + 4], s[kb][8 * t + 5]);
-            pf.w = pack_bf16x2(s[kb][8 * t + 6], s[kb][8 * t + 7]);
-            // the row sum is taken over the rounded probabilities, the values the second MFMA multiplies with
-            l_run = bf16_pair_sum(pf.x, l_run);
-            l_run = bf16_pair_sum(pf.y, l_run);
-            l_run = bf16_pair_sum(pf.z, l_run);
-            l_run = bf16_pair_sum(pf.w, l_run);
-            const u32x4 v0 = *reinterpret_cast<const u32x4 *>(vrow0 + voff0[2 * kb + t]);
-            const u32x4 v1 = *reinterpret_cast<const u32x4 *>(vrow1 + voff1[2 * kb + t]);
-            o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v0),
-                                                          __builtin_bit_cast(bf16x8, pf), o[0], 0, 0, 0);
-            o[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v1),
-                                                          __builtin_bit_cast(bf16x8, pf), o[1], 0, 0, 0);
-        }
+    for (int e = 0; e < 16; e++) {
+        s0[e] -= m;
+        negm[e] = -m;
     }
 }
 
-template <bool FULL>
-__device__ __forceinline__ void attn_stage_resident_nb(int nb, const unsigned char *kp, const unsigned char *vrow0,
-                                                       const unsigned char *vrow1, int vsw0, int vsw1, int key0,
-                                                       int n, int lg, const int (&cs)[4], const u32x4 (&qf)[4],
-                                                       f32x16 (&o)[2], float &m_used, float &l_run, float c)
+// All key blocks of one tile, the number of blocks known at compile time: the pipeline fully unrolled, the two
+// score buffers addressed by constants.  Leaves the halves of the row sum of this lane's keys in l[0] + l[1].
+template <int NBLK>
+__device__ __forceinline__ void att_tile_fixed(const AttnTile &t, const int (&cs)[4], const u32x4 (&qf)[4],
+                                               f32x16 (&o)[2], float &l_run)
 {
-    switch (nb) {
-    case 4: attn_stage_resident<4, FULL>(kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c); break;
-    case 3: attn_stage_resident<3, FULL>(kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c); break;
-    case 2: attn_stage_resident<2, FULL>(kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c); break;
-    default: attn_stage_resident<1, FULL>(kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c); break;
-    }
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    u32x4 kf[4];
+    f32x16 sbuf[2], negm;
+    float l[2] = {0.f, 0.f};
+    o[0] = zero;
+    o[1] = zero;
+    att_first_block(t, cs, NBLK, kf, qf, sbuf[0], negm);
+    const bool partial = (t.n & 31) != 0;           // wave-uniform
+    static_for<NBLK>([&](auto kbc) {
+        constexpr int kb = decltype(kbc)::value;
+        constexpr bool NEXT = kb + 1 < NBLK, NEXT2 = kb + 2 < NBLK;
+        if constexpr (kb == NBLK - 1) {
+            if (partial) att_step<NEXT, NEXT2, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            else att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+        } else {
+            att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+        }
+    });
+    l_run = l[0] + l[1];
 }
 
-__global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_resident_kernel(
+#undef VT_PIN
+
+// ---------------------------------------------------------------------------------------------------------
+// Short key sequences (n <= 288, e.g. 257 tokens at 256 px): one persistent workgroup of eight waves per compute
+// unit walks the (sample, head) items c, c + grid, c + 2 grid, ... with two buffers in LDS, each holding the item's K
+// rows and V rows (128-byte rows, 16-byte chunks XOR-swizzled).  While the first four waves multiply item i out of
+// one buffer (a wave per 32-query tile; the other four join in for samples of more than 128 queries), the second
+// four bring item i+1 into the other buffer by direct loads; one barrier per item.  The staging of an item (its
+// 64 KB come as 128-byte pieces out of 1.5 KB token rows) thus overlaps the arithmetic of the item before it.
+// Vector-memory operations retire in issue order: a wave asks for its first Q tile of the next item right after the
+// prefetch and nothing inside the tile arithmetic depends on either; only a sample with more than eight query
+// tiles (more than 256 queries) loads Q in between.
+// One instantiation per number of 32-key blocks (1 .. 9), so that the tile pipeline is fully unrolled.
+template <int NBLK>
+__global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_kernel(
     const bf16_t *__restrict__ q, int64_t q_rs, int64_t q_hs, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, int64_t kv_bs, int64_t kv_ts, int64_t kv_hs, const int64_t *__restrict__ offsets,
-    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale, int B, int h)
+    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, float scale, int items, int h)
 {
-    constexpr int MAXV = 9;          // 16-byte V chunks per thread: covers n_pad = 288
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int b = blockIdx.x % B, head = blockIdx.x / B;
-    const int64_t row0 = offsets[b];
-    const int Lb = (int)(offsets[b + 1] - row0);
-    if (Lb <= 0) return;
-    const int npad = (n + 31) & ~31;
-    const int vpitch = ((n + 63) & ~63) * 2 + 16;
-    unsigned char *ks = smem;
-    unsigned char *vt = smem + npad * 128;
+    constexpr int NW = 8;                   // waves
+    constexpr int npad = NBLK * 32;         // the host picks the instantiation: NBLK = ceil(n / 32)
+    constexpr int bufsz = 2 * npad * 128;   // K rows, then V rows
+    extern __shared__ __attribute__((aligned(128))) unsigned char smem[];    // rows start on 128-byte boundaries
 
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lg = lane >> 5;
-    const unsigned char *kbase = reinterpret_cast<const unsigned char *>(k + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
-    const unsigned char *vbase = reinterpret_cast<const unsigned char *>(v + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
     const int64_t row_bytes = kv_ts * 2;
+    const float c = scale * 1.44269504088896340736f;
 
-    // Q fragments (B operand of S^T: bytes [32 s + 16 g, +16) of the query row) of this wave's first tile; the
-    // fragments of tile rt + 4 are fetched while tile rt is processed
-    auto load_q = [&](int rt, u32x4 (&dst)[4]) {
+    // Items of this workgroup: blockIdx.x + li * gridDim.x, li = 0, 1, ...; item -> (sample, head) with the heads of a
+    // sample as neighbours, so the pieces of one token row are fetched by workgroups that run at the same time.
+    // First row and query count of every item are put into a small LDS table up front (up to ATT_TBL items per
+    // workgroup; beyond that they are read from `offsets` when needed), so that no step of the loop waits for them.
+    struct Item {
+        int64_t row0;
+        int Lb, b, head;
+    };
+    int64_t *t_row0 = reinterpret_cast<int64_t *>(smem + 2 * bufsz);
+    int *t_len = reinterpret_cast<int *>(t_row0 + ATT_TBL);
+    const int grid = gridDim.x;
+    if ((int)blockIdx.x >= items) return;
+    const int my_items = (items - (int)blockIdx.x + grid - 1) / grid;
+    const bool tabled = my_items <= ATT_TBL;
+    if (tabled) {
+        for (int li = tid; li < my_items; li += 512) {
+            const int b = ((int)blockIdx.x + li * grid) / h;
+            const int64_t r0 = offsets[b];
+            t_row0[li] = r0;
+            t_len[li] = (int)(offsets[b + 1] - r0);
+        }
+    }
+    auto item_of = [&](int li, bool from_table) {
+        Item r;
+        const int it = (int)blockIdx.x + li * grid;
+        r.b = it / h;
+        r.head = it - r.b * h;
+        if (from_table) {
+            const int64_t r0 = t_row0[li];
+            r.row0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(r0 >> 32)) << 32) |
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)r0);
+            r.Lb = __builtin_amdgcn_readfirstlane(t_len[li]);
+        } else {
+            r.row0 = offsets[r.b];
+            r.Lb = (int)(offsets[r.b + 1] - r.row0);
+        }
+        return r;
+    };
+    auto load_q = [&](const Item &im, int rt, u32x4 (&dst)[4]) {
         const int qrow = rt * 32 + lr;
         const unsigned char *qp =
-            reinterpret_cast<const unsigned char *>(q + (row0 + qrow) * q_rs + (int64_t)head * q_hs) + lg * 16;
+            reinterpret_cast<const unsigned char *>(q + (im.row0 + qrow) * q_rs + (int64_t)im.head * q_hs) + lg * 16;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             const u32x4 z = {0u, 0u, 0u, 0u};
-            dst[s] = qrow < Lb ? *reinterpret_cast<const u32x4 *>(qp + s * 32) : z;
+            dst[s] = qrow < im.Lb ? *reinterpret_cast<const u32x4 *>(qp + s * 32) : z;
         }
     };
-    u32x4 qf[4];
-    load_q(wid, qf);
-
-    // K by direct loads (wave-load j covers keys 8j..8j+7), V through registers
-    for (int j = wid; j < npad / 8; j += 4) {
-        const int r = j * 8 + (lane >> 3);
-        const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-        const int key = r < n ? r : n - 1;
-        VT_GLOBAL_TO_LDS(kbase + key * row_bytes + chunk * 16, ks + j * 1024);
-    }
-    u32x4 vreg[MAXV];
+    auto scale_q = [&](u32x4 (&f)[4]) {       // scores come out of the MFMA in log2 units
 #pragma unroll
-    for (int i = 0; i < MAXV; i++) {
-        const int idx = tid + 256 * i;
-        int key = idx >> 3;
-        key = key < n ? key : n - 1;
-        vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + key * row_bytes + (idx & 7) * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < MAXV; i++) {
-        const int idx = tid + 256 * i;
-        const int kr = idx >> 3, ch = idx & 7;
-        if (kr < npad) {
-            // position of key kr in its row: bits 2 and 3 swapped inside the group of 16, group XOR-ed by d >> 4
-            const int kpos = ((kr & ~12) | ((kr & 4) << 1) | ((kr & 8) >> 1)) ^ (16 * ((ch >> 1) & 3));
-            const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint16_t h16 = (uint16_t)(e & 1 ? w[e >> 1] >> 16 : w[e >> 1] & 0xffffu);
-                *reinterpret_cast<uint16_t *>(vt + (ch * 8 + e) * vpitch + kpos * 2) = h16;
-            }
+        for (int s = 0; s < 4; s++) f[s] = att_scale_frag(f[s], c);
+    };
+    // K and V of an item by direct loads, issued by the waves w0, w0 + nw, ...: wave-load j covers rows 8j .. 8j+7 of
+    // K (j < npad / 8) or of V; a lane fetches the 16-byte chunk that belongs at its position of the swizzled row.
+    // Rows past the last key repeat it (their scores are masked).  Issued from assembly: the compiler would
+    // otherwise wait for every direct load in flight before any later read of LDS, i.e. put the prefetch in front
+    // of the arithmetic it is meant to overlap.
+    auto stage_issue = [&](const Item &im, unsigned char *buf, int w0, int nw) {
+        const unsigned char *kbase =
+            reinterpret_cast<const unsigned char *>(k + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
+        const unsigned char *vbase =
+            reinterpret_cast<const unsigned char *>(v + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
+        const int lf = fresh(lane);
+        for (int j = w0; j < 2 * (npad / 8); j += nw) {
+            const bool is_v = j >= npad / 8;
+            const int r = (is_v ? j - npad / 8 : j) * 8 + (lf >> 3);
+            const int chunk = (lf & 7) ^ (is_v ? 2 * (r & 3) : (r >> 1) & 7);
+            const int key = r < n ? r : n - 1;
+            dma16(uniform_ptr(is_v ? vbase : kbase), (uint32_t)(key * row_bytes + chunk * 16),
+                  (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(buf + j * 1024)));
         }
-    }
-    wait_vmcnt<0>();
-    __syncthreads();
+    };
 
     const int sw = (lr >> 1) & 7;
     int cs[4];
 #pragma unroll
     for (int s = 0; s < 4; s++) cs[s] = ((2 * s + lg) ^ sw) * 16;
-    const float c = scale * 1.44269504088896340736f;
-    const int nblk = npad / 32;
-    const int nstage = (nblk + 3) / 4;
-    const int nbs = (nblk + nstage - 1) / nstage;          // blocks per stage (the last stage takes the rest)
-    const unsigned char *vrow0 = vt + lr * vpitch + lg * 16;
-    const unsigned char *vrow1 = vt + (32 + lr) * vpitch + lg * 16;
-    const int vsw0 = 16 * ((lr >> 4) & 3), vsw1 = 16 * ((2 + (lr >> 4)) & 3);
 
-    for (int rt = wid; rt * 32 < Lb; rt += 4) {
-        const int qrow = rt * 32 + lr;
-        const bool row_live = qrow < Lb;
-        u32x4 qn[4];
-        load_q(rt + 4, qn);            // zeros past the last tile
-        f32x16 o[2];
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) o[i][e] = 0.f;
-        float m_used = -INFINITY, l_run = 0.f;
-        for (int st = 0; st < nstage; st++) {
-            const int key0 = st * nbs * 32;
-            const int nb = st + 1 < nstage ? nbs : nblk - st * nbs;
-            const unsigned char *kp = ks + (key0 + lr) * 128;
-            if (key0 + nb * 32 <= n)
-                attn_stage_resident_nb<true>(nb, kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c);
-            else
-                attn_stage_resident_nb<false>(nb, kp, vrow0, vrow1, vsw0, vsw1, key0, n, lg, cs, qf, o, m_used, l_run, c);
+    Item cur = item_of(0, false);
+    stage_issue(cur, smem, wid, NW);
+    u32x4 qf[4], qn[4];
+    load_q(cur, wid, qf);
+    wait_vmcnt<0>();
+    __syncthreads();
+    Item nxt = cur;
+    if (my_items > 1) nxt = item_of(1, tabled);
+
+    for (int li = 0, par = 0; li < my_items; li++, par ^= 1) {
+        unsigned char *buf = smem + par * bufsz;
+        const bool has_next = li + 1 < my_items;
+        // The second half of the waves has a tile only in samples of more than 128 queries: it issues the prefetch
+        // of the next item, the first half goes straight to its tiles.  Every wave then asks for its first Q tile of
+        // the next item; nothing in the tile arithmetic depends on these loads.
+        if (has_next) {
+            if (wid >= NW / 2) stage_issue(nxt, smem + (par ^ 1) * bufsz, wid - NW / 2, NW / 2);
+            load_q(nxt, wid, qn);
         }
-        const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
-        if (row_live) attn_store(out + (row0 + qrow) * o_rs + (int64_t)head * o_hs, o, l_tot, lg);
+        const AttnTile tile = {buf + lr * 128, att_v_lane(buf + npad * 128, lane), n, lg};
+        for (int rt = wid; rt * 32 < cur.Lb; rt += NW) {
+            const int qrow = rt * 32 + lr;
+            if (rt != wid) {        // a ninth tile and beyond (more than 256 queries): waits behind the prefetch
+                load_q(cur, rt, qf);
+                wait_vmcnt<0>();    // here, so that the common path carries no pending load into the arithmetic
+            }
+            f32x16 o[2];
+            float l_run;
+            scale_q(qf);
+            att_tile_fixed<NBLK>(tile, cs, qf, o, l_run);
+            const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+            if (qrow < cur.Lb) attn_store(out + (cur.row0 + qrow) * o_rs + (int64_t)cur.head * o_hs, o, l_tot, lg);
+        }
+        cur = nxt;
+        if (li + 2 < my_items) nxt = item_of(li + 2, tabled);
+        // The waves that issued direct loads wait for them here (the compiler does not know of them); stores count
+        // in the same queue, so a wave that has just stored a tile would wait for that too: the first half of the
+        // waves, which stores in every item, has issued no direct load and needs no wait of its own - the compiler
+        // places the wait for the Q loads where they are used.
+        if (wid >= NW / 2) wait_vmcnt<0>();
 #pragma unroll
         for (int s = 0; s < 4; s++) qf[s] = qn[s];
+        __syncthreads();      // the next item's buffer is complete; this item's buffer is free
     }
 }
 
@@ -452,14 +627,33 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
                               int64_t o_hs, int B, int h, int n, int max_rows, float scale, hipStream_t st)
 {
     if (n <= 288) {
+        // keys and values resident in LDS: one persistent workgroup per compute unit, two buffers of K rows + V rows
         const int npad = (n + 31) & ~31;
-        const size_t lds_r = (size_t)npad * 128 + 64 * ((size_t)((n + 63) & ~63) * 2 + 16);
-        auto kern_r = sparse_attention_bf16_d64_resident_kernel;
-        VT_RESERVE_LDS(kern_r, 80 * 1024, "sparse_attention");
-        dim3 grid_r((unsigned)(B * h)), block_r(256);
-        kern_r<<<grid_r, block_r, lds_r, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v,
-                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale, B, h);
-        return check_launch("sparse_attention");
+        const size_t lds_p = 4 * (size_t)npad * 128 + ATT_TBL * 12;       // + the item table
+        const int items = B * h;
+        const int cus = compute_units();
+        dim3 grid_p((unsigned)(items < cus ? items : cus)), block_p(512);
+#define VT_ATT_PIPE(NB)                                                                                            \
+    case NB: {                                                                                                     \
+        auto kern_p = sparse_attention_bf16_d64_pipelined_kernel<NB>;                                              \
+        VT_RESERVE_LDS(kern_p, 160 * 1024, "sparse_attention");                                                    \
+        kern_p<<<grid_p, block_p, lds_p, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v, \
+                                               kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale,  \
+                                               items, h);                                                          \
+        return check_launch("sparse_attention");                                                                   \
+    }
+        switch (npad / 32) {
+            VT_ATT_PIPE(1)
+            VT_ATT_PIPE(2)
+            VT_ATT_PIPE(3)
+            VT_ATT_PIPE(4)
+            VT_ATT_PIPE(5)
+            VT_ATT_PIPE(6)
+            VT_ATT_PIPE(7)
+            VT_ATT_PIPE(8)
+            VT_ATT_PIPE(9)
+        }
+#undef VT_ATT_PIPE
     }
     const size_t lds = 2 * (size_t)ABUF;
     const int qchunks = (int)ceil_div(max_rows, AQ);

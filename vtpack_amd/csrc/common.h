@@ -14,6 +14,7 @@ namespace vtdge {
 // ---------------------------------------------------------------- errors
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+int compute_units();      // of the current device (256 on an MI355X)
 
 #define VT_REQUIRE(cond, code, ...)  \
     do {                             \
@@ -150,6 +151,14 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t l
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base)
                  : "memory", "m0");
+}
+// a wave-uniform pointer as the scalar register pair an address operand of the direct loads needs
+__device__ __forceinline__ const void *uniform_ptr(const void *p)
+{
+    const uint64_t u = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+    return reinterpret_cast<const void *>((uintptr_t)(((uint64_t)hi << 32) | lo));
 }
 // the same with a compile-time byte offset (0 .. 4095) added to the global address.  The instruction adds its
 // immediate to the LDS address too, so that is lowered by as much first: lds_addr must be at least IMM.

@@ -23,6 +23,22 @@ int check_launch(const char *what)
     return VTDGE_OK;
 }
 
+int compute_units()
+{
+    // asked once per device; the answer cannot change while the process lives
+    static std::once_flag once[16];
+    static int count[16];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
+    std::call_once(once[dev], [&] {
+        hipDeviceProp_t prop;
+        count[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0
+                         ? prop.multiProcessorCount
+                         : 256;
+    });
+    return count[dev];
+}
+
 }  // namespace vtdge
 
 extern "C" int vtdge_version(void) { return 100; }
