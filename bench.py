@@ -86,6 +86,8 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
     if name == "vtdge_decompress_layernorm":
         return f"decompress_ln_kernel<{T}, {b(tag[1])}, {gs(tag[2])}>"
+    if name == "vtdge_decompress_router":
+        return f"decompress_route_kernel<{T}, {gs(tag[3])}, {b(tag[1])}>"
     if name == "vtdge_layernorm":
         nv = tag[3] * esz // 16                           # 16-byte vectors per row
         return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
@@ -136,6 +138,9 @@ def algorithmic_work(name, tag, esz, geo):
         return "hbm", B * N * C * esz + 32 * L + L * C * esz * (2 if tag[1] else 1)
     if name == "vtdge_decompress":
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + (2 if tag[2] else 1) * B * N * C * esz
+    if name == "vtdge_decompress_router":
+        # the scatter-back's bytes: routing the next block reads nothing more (gate indices in, logits out: KBs)
+        return "hbm", (2 if tag[1] else 1) * L * C * esz + 2 * B * N * C * esz + 16 * B * geo["regions"]
     if name == "vtdge_decompress_layernorm":
         # the scatter-back plus one more write of every token (the next block's first LayerNorm)
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + 3 * B * N * C * esz
@@ -258,7 +263,7 @@ def run_model_workload(args, torch):
         st["seconds"] += sec
         st["work"] += amount
         st["bytes"] += rest[0] if rest else 0.0
-        if name == "vtdge_decompress":
+        if name in ("vtdge_decompress", "vtdge_decompress_router", "vtdge_decompress_layernorm"):
             blk += 1
     kernels = {}
     for sym, st in stats.items():

@@ -125,6 +125,20 @@ int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *p
                                const void *ln_bias, float ln_eps, int B, int N, int C, int W, int extra, int dtype,
                                void *stream);
 
+/* Scatter back by region, and the NEXT block's router on the tokens just written:
+ *   out[b,t,:] = (in[row,:] - sub[row,:]) + ref[b,t,:]        (as vtdge_decompress with `sub` and `ref`; sub nullable)
+ *   next_gate [B, H/R, W/R, S2], next_indices int64 [B, H/R, W/R] = vtdge_router(out, next_weight, next_bias)
+ * i.e. the last step of one block (vtpack/layers/dge.py:87-112) together with DynamicRouter.forward + argmax of the
+ * block that follows (vtpack/layers/dge.py:145-150, :75), which would read the same tokens back.  The packed rows
+ * are found from this block's gate indices `cur_indices` [B, H/R, W/R] (S splits in `splits`, as given to
+ * vtdge_index_to_patch) and `offsets` [B+1] instead of the patch list.  Both results are bit-identical to the two
+ * separate calls.  next_weight == NULL (with next_bias, next_indices) leaves the router out.  R must be 4 and every
+ * split size must divide it; VTDGE_ERR_UNSUPPORTED for another R. */
+int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits,
+                            const int64_t *offsets, const void *ref, void *out, const void *next_weight,
+                            const void *next_bias, void *next_gate, int64_t *next_indices, int B, int H, int W, int C,
+                            int extra, int R, int S, int S2, int dtype, void *stream);
+
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */
 int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out, const int64_t *rows_dev,

@@ -554,3 +554,35 @@ def test_batched_sparse_gemm(dev, dtype, ta, tb):
         else:
             # bf16 output of sums of ~64 products of N(0,1) values: one bf16 rounding of |x| <~ 40
             assert rel_err(got.float(), want) <= 2 ** -8
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,Hr,Wr,C,extra", [(5, 4, 4, 384, 1), (3, 8, 8, 192, 1), (4, 3, 5, 64, 0), (2, 4, 4, 768, 2),
+                                               (2, 14, 14, 64, 0), (3, 2, 2, 128, 1)])
+def test_scatter_back_with_the_next_router(dev, dtype, B, Hr, Wr, C, extra):
+    """The scatter-back by region that also routes the next block: the tokens, the next gate logits and the next
+    gate indices equal those of the two separate operators bit for bit (which the oracle pins), for every split
+    mix, width (one and several regions per wave, several vectors per lane) and count of extra tokens."""
+    from vtpack_amd import ops
+    H, W = 4 * Hr, 4 * Wr
+    g = torch.Generator().manual_seed(B * 100 + C + extra)
+    idx = torch.from_numpy(random_indices(B + C, B, Hr, Wr)).to(dev)
+    splits = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    patches, offsets, lengths = ops.index_to_patch(idx, splits, 4, extra)
+    L = int(offsets[-1])
+    q = torch.randn(L, C, generator=g).to(dtype).to(dev)
+    comp = torch.randn(L, C, generator=g).to(dtype).to(dev)
+    x = torch.randn(B, extra + H * W, C, generator=g).to(dtype).to(dev)
+    wgt = (torch.randn(3, C, generator=g) / C ** 0.5).to(dtype).to(dev)
+    bias = (torch.randn(3, generator=g) * 0.1).to(dtype).to(dev)
+    for sub in (comp, None):
+        want = ops.decompress(q, patches[:L], x, W, extra, add_ref=True, sub=sub)
+        want_gate, want_idx = ops.router(want, wgt, bias, H, W, 4)
+        got, gate, nidx = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt,
+                                                next_bias=bias)
+        assert torch.equal(got, want)
+        assert torch.equal(nidx, want_idx) and torch.equal(gate, want_gate)
+    # without a next router it is the plain scatter-back
+    alone, g0, i0 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp)
+    assert g0 is None and i0 is None
+    assert torch.equal(alone, ops.decompress(q, patches[:L], x, W, extra, add_ref=True, sub=comp))

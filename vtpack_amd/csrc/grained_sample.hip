@@ -760,6 +760,165 @@ __global__ __launch_bounds__(256) void decompress_ln_kernel(const T *__restrict_
     }
 }
 
+// ------------------------------------------------- decompress + next router
+// Scatter back by REGION instead of by packed row, so that the same wave can route the next block: a group of GS
+// lanes owns one R x R region (R = 4) of one sample.  The packed rows of a region are consecutive (regions in
+// row-major order, sub-patches in row-major order inside a region), starting at
+//   offsets[b] + extra + sum of the query counts of the sample's earlier regions,
+// which the group adds up from the gate indices itself.  It writes out = (in - sub) + ref for the region's 16
+// tokens (the same arithmetic and rounding as decompress_kernel), sums the values as stored, in the order the
+// router sums them, and finishes with the router's Linear + argmax on the NEXT block's gate weights: the indices
+// and logits it leaves are bit for bit those of router_kernel run on `out`, without a second pass over the tokens.
+// The group of a sample's first region also scatters the sample's extra tokens.
+template <typename T, int PS, bool SUB>
+__device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T *__restrict__ sub, int64_t r0,
+                                               const T *__restrict__ refp, T *__restrict__ outp, int W, int C,
+                                               float (&acc)[Elem<T>::VEC])
+{
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int STEP = 4 / PS;
+#pragma unroll 1
+    for (int dy = 0; dy < 4; dy++) {                       // one token row (4 tokens) at a time; not unrolled: the
+                                                           // loads of one row are what a wave keeps in flight
+        constexpr int NJ = PS;                              // packed rows these tokens take their values from
+        const int j0 = (dy / STEP) * PS;
+        u32x4 xr[4], ir[NJ], sr[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            ir[j] = *reinterpret_cast<const u32x4 *>(in + (r0 + j0 + j) * (int64_t)C);
+            if constexpr (SUB) sr[j] = *reinterpret_cast<const u32x4 *>(sub + (r0 + j0 + j) * (int64_t)C);
+        }
+#pragma unroll
+        for (int dx = 0; dx < 4; dx++)
+            xr[dx] = *reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C);
+        // in - sub, rounded to the storage type (kept packed: four registers per row)
+        if constexpr (SUB) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                float dv[VEC], sv[VEC];
+                Elem<T>::unpack(ir[j], dv);
+                Elem<T>::unpack(sr[j], sv);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) dv[c] -= sv[c];
+                ir[j] = Elem<T>::pack(dv);
+            }
+        }
+#pragma unroll
+        for (int dx = 0; dx < 4; dx++) {
+            float r[VEC], dv[VEC];
+            Elem<T>::unpack(xr[dx], r);
+            Elem<T>::unpack(ir[dx / STEP], dv);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) r[c] += dv[c];
+            const u32x4 packed = Elem<T>::pack(r);
+            *reinterpret_cast<u32x4 *>(outp + ((int64_t)dy * W + dx) * C) = packed;
+            float f[VEC];
+            Elem<T>::unpack(packed, f);                   // as stored: what the next block's router reads
+#pragma unroll
+            for (int c = 0; c < VEC; c++) acc[c] += f[c];
+        }
+    }
+}
+
+template <typename T, int GS, bool SUB>
+__global__ __launch_bounds__(256) void decompress_route_kernel(
+    const T *__restrict__ in, const T *__restrict__ sub, const int64_t *__restrict__ cur_indices,
+    const int64_t *__restrict__ splits, const int64_t *__restrict__ offsets, const T *__restrict__ ref,
+    T *__restrict__ out, const T *__restrict__ weight, const T *__restrict__ bias, T *__restrict__ gate,
+    int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2)
+{
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int R = 4;
+    const int lane = threadIdx.x & (GS - 1);
+    const int Hr = H / R, Wr = W / R, nreg = Hr * Wr;
+    const int64_t region = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
+    if (region >= (int64_t)B * nreg) return;
+    const int b = (int)(region / nreg);
+    const int rr = (int)(region % nreg);
+    const int ry = rr / Wr, rx = rr % Wr;
+    const int N = extra + H * W;
+    const int nvec = C / VEC;
+
+    auto split_of = [&](int64_t reg) {
+        int64_t g = cur_indices[reg];
+        g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+        return (int)splits[g];
+    };
+    // first packed row of this region (query counts are small integers: exact in fp32)
+    float before = 0.f;
+    for (int r2 = lane; r2 < rr; r2 += GS) {
+        const int ps2 = split_of((int64_t)b * nreg + r2);
+        before += (float)(ps2 * ps2);
+    }
+    const int64_t row_b = offsets[b];
+    const int64_t r0 = row_b + extra + (int64_t)group_sum<GS>(before);
+    int ps = split_of(region);
+    if constexpr (GS == WAVE) ps = __builtin_amdgcn_readfirstlane(ps);      // one region per wave: a scalar branch
+
+    float part[VTDGE_MAX_SPLITS];
+#pragma unroll
+    for (int s = 0; s < VTDGE_MAX_SPLITS; s++) part[s] = 0.f;
+    const int64_t tok0 = (int64_t)(ry * R) * W + rx * R + extra;
+    for (int v = lane; v < nvec; v += GS) {
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+        const int64_t off = ((int64_t)b * N + tok0) * C + v * VEC;
+        const T *inv = in + v * VEC;
+        const T *subv = SUB ? sub + v * VEC : nullptr;
+        if (ps == 4) region_scatter<T, 4, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
+        else if (ps == 2) region_scatter<T, 2, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
+        else region_scatter<T, 1, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
+        if (rr == 0) {          // the sample's extra tokens: packed rows row_b .. row_b + extra - 1
+            for (int e = 0; e < extra; e++) {
+                float d[VEC], r[VEC];
+                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(inv + (row_b + e) * (int64_t)C), d);
+                if constexpr (SUB) {
+                    float sv[VEC];
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(subv + (row_b + e) * (int64_t)C), sv);
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) d[c] -= sv[c];
+                    Elem<T>::unpack(Elem<T>::pack(d), d);      // rounded to the storage type
+                }
+                const int64_t oe = ((int64_t)b * N + e) * C + v * VEC;
+                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + oe), r);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) r[c] += d[c];
+                *reinterpret_cast<u32x4 *>(out + oe) = Elem<T>::pack(r);
+            }
+        }
+        if (weight != nullptr) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) acc[i] = Elem<T>::round(acc[i] / (float)(R * R));
+#pragma unroll
+            for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
+                if (s < S2) {
+                    float w[VEC];
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(weight + (int64_t)s * C + v * VEC), w);
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) part[s] += acc[i] * w[i];
+                }
+            }
+        }
+    }
+    if (weight == nullptr) return;
+    float best = 0.f;
+    int best_s = 0;
+#pragma unroll
+    for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
+        if (s < S2) {
+            float logit = group_sum<GS>(part[s]) + Elem<T>::load(bias + s);
+            logit = Elem<T>::round(logit);
+            if (gate != nullptr && lane == 0) Elem<T>::store(gate + region * S2 + s, logit);
+            if (s == 0 || logit > best) {  // strict >: lowest index wins a tie
+                best = logit;
+                best_s = s;
+            }
+        }
+    }
+    if (lane == 0) indices[region] = best_s;
+}
+
 // --------------------------------------------------------------- layernorm
 constexpr int LN_RPW = 4;   // rows per wave: their loads are issued together so that enough bytes are in flight
 
@@ -1074,6 +1233,43 @@ extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const
 #undef VT_DISPATCH
 #undef VT_LAUNCH
     return check_launch("decompress_layernorm");
+}
+
+extern "C" int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices,
+                                       const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
+                                       const void *next_weight, const void *next_bias, void *next_gate,
+                                       int64_t *next_indices, int B, int H, int W, int C, int extra, int R, int S,
+                                       int S2, int dtype, void *stream)
+{
+    VT_REQUIRE(in && cur_indices && splits && offsets && ref && out, VTDGE_ERR_ARG, "decompress_router: NULL operand");
+    VT_REQUIRE((next_weight == nullptr) == (next_bias == nullptr) && (next_weight == nullptr) == (next_indices == nullptr),
+               VTDGE_ERR_ARG, "decompress_router: the next router needs weight, bias and indices together");
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && extra >= 0, VTDGE_ERR_ARG, "decompress_router: bad sizes");
+    VT_REQUIRE(R == 4, VTDGE_ERR_UNSUPPORTED, "decompress_router: region size %d (4 only)", R);
+    VT_REQUIRE(H % R == 0 && W % R == 0, VTDGE_ERR_ARG, "decompress_router: H=%d, W=%d not multiples of region %d", H,
+               W, R);
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS && S2 >= 1 && S2 <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED,
+               "decompress_router: split counts %d / %d outside [1,%d]", S, S2, VTDGE_MAX_SPLITS);
+    if (int rc = check_channels(C, dtype, "decompress_router")) return rc;
+    VT_REQUIRE(aligned16(in) && aligned16(sub) && aligned16(ref) && aligned16(out) && aligned16(next_weight),
+               VTDGE_ERR_ARG, "decompress_router: operands must be 16-byte aligned");
+    const int64_t regions = (int64_t)B * (H / R) * (W / R);
+    const int gs = group_size(C / (dtype == VTDGE_BF16 ? 8 : 4));
+    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
+    hipStream_t st = (hipStream_t)stream;
+#define VT_LAUNCH2(T, GS, SUBF)                                                                                    \
+    decompress_route_kernel<T, GS, SUBF><<<grid, block, 0, st>>>(                                                  \
+        (const T *)in, (const T *)sub, cur_indices, splits, offsets, (const T *)ref, (T *)out,                     \
+        (const T *)next_weight, (const T *)next_bias, (T *)next_gate, next_indices, B, H, W, C, extra, S, S2)
+#define VT_LAUNCH(T, GS) do { if (sub) VT_LAUNCH2(T, GS, true); else VT_LAUNCH2(T, GS, false); } while (0)
+#define VT_GROUP(T) \
+    do { if (gs == 64) VT_LAUNCH(T, 64); else if (gs == 32) VT_LAUNCH(T, 32); else if (gs == 16) VT_LAUNCH(T, 16); \
+         else VT_LAUNCH(T, 8); } while (0)
+    if (dtype == VTDGE_F32) VT_GROUP(float); else VT_GROUP(bf16_t);
+#undef VT_GROUP
+#undef VT_LAUNCH
+#undef VT_LAUNCH2
+    return check_launch("decompress_router");
 }
 
 extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,

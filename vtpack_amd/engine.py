@@ -27,6 +27,10 @@ FUSE_NEXT_NORM = False
 # whole region with nothing to overlap the three phases (30 us against 22 us for the two kernels side by side at the
 # headline config), and both chains of the block wait for it.
 FUSE_ROUTER_NORM = False
+# The scatter-back of a block can route the next block on the tokens it has just written (by region instead of by
+# packed row: `vtdge_decompress_router`): the next block's router kernel and its pass over x disappear, and with it
+# the first kernel of the routing chain, the longer of the two chains.  On by default (same bits as the two kernels).
+FUSE_NEXT_ROUTER = True
 
 
 def _side_stream(device, slot=0):
@@ -85,27 +89,33 @@ def _key_value_source(attn, x_ln, H, W, extra):
     return ops.layernorm(red, attn.norm.weight, attn.norm.bias, attn.norm.eps).view(B, -1, C)
 
 
-def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=None):
+def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_block=None):
     """x [B, N, C] -> [B, N, C] for a DGE transformer block (`models.dge.deit_dge.Block` or
     `models.dge.pvt_dge.Block`) in eval mode.
 
     `gate` [B, Hr, Wr, S] overrides the router's logits (used by the parity tests).
     `overlap` issues the key/value chain on a second stream next to the routing chain.
-    `x_ln` is norm1(x) when the caller already has it; `next_norm` is the LayerNorm the next block applies to this
-    block's output first: the scatter-back kernel then writes that too and the call returns (out, next_norm(out)).
+    `next_block` is the block that runs next on this block's output (same token grid): the call then returns
+    (out, carry), where `carry` holds what this block has already worked out for it - the next block's gate logits and
+    indices from the scatter-back kernel (`FUSE_NEXT_ROUTER`), or its first LayerNorm (`FUSE_NEXT_NORM`) - to be
+    passed to the next call as `carry`.
     """
     dge, attn, mlp = block.dge, block.attn, block.mlp
     B, N, C = x.shape
     extra = N - H * W
     R = dge.region_size
     x = x.contiguous()
+    carry = carry or {}
+    x_ln = carry.get("x_ln")
+    routed = carry.get("routed") if gate is None else None
 
     n1, n2 = block.norm1, block.norm2
     overlap = overlap and OVERLAP
     main = torch.cuda.current_stream(x.device)
     side = _side_stream(x.device, main.cuda_stream) if overlap else main
 
-    fuse_rn = FUSE_ROUTER_NORM and gate is None and x_ln is None and ops.fits_router_layernorm(x, R)
+    fuse_rn = (FUSE_ROUTER_NORM and gate is None and routed is None and x_ln is None
+               and ops.fits_router_layernorm(x, R))
     if fuse_rn:
         gate, indices, x_ln = ops.router_layernorm(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R,
                                                    n1.weight, n1.bias, n1.eps)
@@ -120,7 +130,9 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
         kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)                 # [B, n, 2C] = [B, n, 2, h, d]
 
     # routing chain (caller's stream)
-    if not fuse_rn:
+    if routed is not None:
+        gate, indices = routed
+    elif not fuse_rn:
         if gate is None:
             gate, indices = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
         else:
@@ -143,10 +155,16 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
     hid = ops.linear(q1_ln, mlp.fc1.weight, mlp.fc1.bias, act="gelu", rows_dev=rows_dev)
     q2 = ops.linear(hid, mlp.fc2.weight, mlp.fc2.bias, residual=q1, rows_dev=rows_dev)
 
-    out_ln = None
-    if next_norm is not None and FUSE_NEXT_NORM and ops.fits_decompress_layernorm(x):
-        out, out_ln = ops.decompress_layernorm(q2, patches, x, W, extra, next_norm.weight, next_norm.bias,
-                                               next_norm.eps, sub=comp, rows_dev=rows_dev, rows=cap)
+    handed = {}
+    nxt = next_block.dge if next_block is not None else None
+    if nxt is not None and FUSE_NEXT_NORM and ops.fits_decompress_layernorm(x):
+        nn1 = next_block.norm1
+        out, handed["x_ln"] = ops.decompress_layernorm(q2, patches, x, W, extra, nn1.weight, nn1.bias, nn1.eps,
+                                                       sub=comp, rows_dev=rows_dev, rows=cap)
+    elif nxt is not None and FUSE_NEXT_ROUTER and R == 4 and nxt.region_size == 4:
+        out, ngate, nidx = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
+                                                 next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias)
+        handed["routed"] = (ngate, nidx)
     else:
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 
@@ -165,9 +183,20 @@ def block_forward(block, x, H, W, gate=None, overlap=True, x_ln=None, next_norm=
     dge.states.update({"comp": Deferred(cut(comp)), "input": x, "patches": Deferred(cut(patches)),
                        "batches": Deferred(batches), "batches_device": lengths, "offsets_device": offsets,
                        "gate": gate, "size": (H, W), "num_extra_tokens": extra, "queries": Deferred(cut(q2))})
-    if next_norm is not None:
-        return out, out_ln          # out_ln is None when the fused kernel does not apply: the next block normalises
+    if next_block is not None:
+        return out, handed
     return out
+
+
+def _run_blocks(blocks, x, H, W):
+    """A chain of blocks on one token grid, each handing the next what it has already computed for it."""
+    carry = None
+    for i, blk in enumerate(blocks):
+        if i + 1 < len(blocks):
+            x, carry = block_forward(blk, x, H, W, carry=carry, next_block=blocks[i + 1])
+        else:
+            x = block_forward(blk, x, H, W, carry=carry)
+    return x
 
 
 def model_forward(model, images):
@@ -193,13 +222,7 @@ def model_forward(model, images):
     for e, t in enumerate(front):
         x[:, e:e + 1, :] = t
     x += model.pos_embed
-    x_ln = None
-    blocks = list(model.blocks)
-    for i, blk in enumerate(blocks):
-        if i + 1 < len(blocks):     # the scatter-back of this block also writes the next block's norm1
-            x, x_ln = block_forward(blk, x, G, G, x_ln=x_ln, next_norm=blocks[i + 1].norm1)
-        else:
-            x = block_forward(blk, x, G, G, x_ln=x_ln)
+    x = _run_blocks(list(model.blocks), x, G, G)
     nrm = model.norm
 
     def head(lin, t):
@@ -254,13 +277,7 @@ def pvt_forward(model, images):
             x += pos
         else:
             x = tok + model._get_pos_embed(pos, pe, H, W)
-        x_ln = None
-        blocks = list(getattr(model, f"block{i + 1}"))
-        for bi, blk in enumerate(blocks):
-            if bi + 1 < len(blocks):
-                x, x_ln = block_forward(blk, x, H, W, x_ln=x_ln, next_norm=blocks[bi + 1].norm1)
-            else:
-                x = block_forward(blk, x, H, W, x_ln=x_ln)
+        x = _run_blocks(list(getattr(model, f"block{i + 1}")), x, H, W)
         if not last:
             outputs[f"res{i + 2}"] = x.view(B, H, W, C)
         elif model.num_classes == 0:

@@ -174,6 +174,44 @@ def decompress_layernorm(inp, patches, reference, width, num_extra_tokens, ln_we
     return out, ln_out
 
 
+def decompress_router(inp, indices, splits, offsets, reference, H, W, region_size, sub=None, next_weight=None,
+                      next_bias=None, want_gate=True):
+    """Scatter (inp - sub) + reference back over the tokens by region, and route the NEXT block on the result:
+    -> (out, next_gate or None, next_indices or None).  `indices` [B, Hr, Wr] are this block's gate indices, `offsets`
+    [B+1] the prefix of its query counts.  The three outputs equal decompress(...) and router(out, next_weight,
+    next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75."""
+    _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
+    inp, reference = _contig(inp), _contig(reference)
+    sub = None if sub is None else _contig(sub)
+    indices, splits = _contig(indices), _contig(splits)
+    B, N, C = reference.shape
+    extra = N - H * W
+    _check_like(inp, reference=reference, sub=sub, next_weight=next_weight, next_bias=next_bias)
+    if inp.shape[-1] != C or (sub is not None and sub.shape != inp.shape):
+        raise ValueError("packed rows do not match the reference's channel count")
+    if indices.dtype != torch.int64 or splits.dtype != torch.int64 or offsets.dtype != torch.int64:
+        raise TypeError("indices, splits and offsets must be int64")
+    if extra < 0 or H % region_size or W % region_size or tuple(indices.shape) != (B, H // region_size, W // region_size):
+        raise ValueError(f"gate indices {tuple(indices.shape)} do not match a {H}x{W} grid of regions of {region_size}")
+    if offsets.numel() != B + 1:
+        raise ValueError("offsets must have B + 1 entries")
+    out = torch.empty((B, N, C), dtype=inp.dtype, device=inp.device)
+    S = splits.numel()
+    gate = nidx = None
+    S2 = S
+    if next_weight is not None:
+        next_weight, next_bias = _contig(next_weight), _contig(next_bias)
+        S2 = next_weight.shape[0]
+        _check_router(next_weight, next_bias, C, S2, extra, H, W, region_size)
+        Hr, Wr = H // region_size, W // region_size
+        gate = torch.empty((B, Hr, Wr, S2), dtype=inp.dtype, device=inp.device) if want_gate else None
+        nidx = torch.empty((B, Hr, Wr), dtype=torch.int64, device=inp.device)
+    call("vtdge_decompress_router", ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference),
+         ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), B, H, W, C, extra, region_size, S, S2,
+         dtype_code(inp), stream_ptr(), tag=("decompress_router", sub is not None, next_weight is not None, C))
+    return out, gate, nidx
+
+
 def fits_decompress_layernorm(x):
     """Whether a row of x is at most 64 16-byte vectors (the fused scatter + LayerNorm holds a row in one wave)."""
     return x.shape[-1] * x.element_size() <= 64 * 16
