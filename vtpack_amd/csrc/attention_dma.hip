@@ -13,87 +13,7 @@
 
 namespace vtdge {
 
-constexpr int AQ = 128;    // query rows per workgroup (4 waves x 32)
-constexpr int AK = 128;    // keys per stage
-constexpr int AVP = AK * 2 + 16;                    // V^T row pitch (bytes)
-constexpr int ABUF = AK * 128 + 64 * AVP;           // one K + V^T buffer
-
-// One stage of up to 128 keys for a wave's 32 queries (online softmax update + O^T += V^T P^T).
-//   ks: first K row of the stage in LDS (128-byte rows, XOR-swizzled chunks);  vt: V^T base in LDS, rows of
-//   `vpitch` bytes whose key columns start at `vcol`;  key0: index of the stage's first key;  FULL: all 128 exist.
-template <bool FULL>
-__device__ __forceinline__ void attn_stage(const unsigned char *ks, const unsigned char *vt, int vpitch, int vcol,
-                                           int key0, int n, int lr, int lg, const int (&cs)[4], const u32x4 (&qf)[4],
-                                           f32x16 (&o)[2], float &m_run, float &l_run, float c)
-{
-    const int nb = FULL ? 4 : (n - key0 + 31) / 32;
-    int vsw[2];                                                  // key-group swizzle of this lane's two V^T rows
-#pragma unroll
-    for (int db = 0; db < 2; db++) vsw[db] = 8 * (((db * 32 + lr) >> 4) & 3);
-    f32x16 s[4];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int kb = 0; kb < 4; kb++) {
-        if (FULL || kb < nb) {
-#pragma unroll
-            for (int e = 0; e < 16; e++) s[kb][e] = 0.f;
-            const unsigned char *kp = ks + (kb * 32 + lr) * 128;
-#pragma unroll
-            for (int sl = 0; sl < 4; sl++) {
-                const u32x4 kf = *reinterpret_cast<const u32x4 *>(kp + cs[sl]);
-                Slab<bf16_t>::mma(kf, qf[sl], s[kb]);
-            }
-            if constexpr (!FULL) {
-#pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    const int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
-                    if (key >= n) s[kb][e] = -INFINITY;
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < 16; e++) mx = fmaxf(mx, s[kb][e]);
-        }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(m_run, mx * c);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
-    l_run *= alpha;
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) o[i][e] *= alpha;
-#pragma unroll
-    for (int kb = 0; kb < 4; kb++) {
-        if (FULL || kb < nb) {
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], c, -m_new));
-                s[kb][e] = p;
-                l_run += p;
-            }
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                u32x4 pf;
-                pf.x = pack_bf16x2(s[kb][8 * t + 0], s[kb][8 * t + 1]);
-                pf.y = pack_bf16x2(s[kb][8 * t + 2], s[kb][8 * t + 3]);
-                pf.z = pack_bf16x2(s[kb][8 * t + 4], s[kb][8 * t + 5]);
-                pf.w = pack_bf16x2(s[kb][8 * t + 6], s[kb][8 * t + 7]);
-#pragma unroll
-                for (int db = 0; db < 2; db++) {
-                    const unsigned char *vp = vt + (db * 32 + lr) * vpitch + vcol * 2;
-                    const int k0 = kb * 32 + 16 * t + 4 * lg;
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp + ((k0) ^ vsw[db]) * 2);
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + ((k0 + 8) ^ vsw[db]) * 2);
-                    u32x4 vf;
-                    vf.x = lo.x; vf.y = lo.y; vf.z = hi.x; vf.w = hi.y;
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                                   __builtin_bit_cast(bf16x8, pf), o[db], 0, 0, 0);
-                }
-            }
-        }
-    }
-}
+constexpr int AQ = 128;    // query rows per workgroup of the streaming kernel (4 waves x 32)
 
 // normalise and store this lane's query row
 __device__ __forceinline__ void attn_store(bf16_t *op, const f32x16 (&o)[2], float l_tot, int lg)
@@ -312,7 +232,7 @@ __device__ __forceinline__ void att_first_block(const AttnTile &t, const int (&c
 #pragma unroll
         for (int sl = 0; sl < 4; sl++) kf[sl] = att_read_k(t, cs, 1, sl);
     }
-    if (nblk == 1 && (t.n & 31) != 0) {        // a lone, partial block: its missing keys must not set the reference
+    if (nblk == 1 && t.n < 32) {               // a lone, partial block: its missing keys must not set the reference
         const int lim = t.n - 4 * t.lg;
 #pragma unroll
         for (int e = 0; e < 16; e++)
@@ -352,6 +272,54 @@ __device__ __forceinline__ void att_tile_fixed(const AttnTile &t, const int (&cs
         }
     });
     l_run = l[0] + l[1];
+}
+
+// One stage of NB key blocks of a sequence that is streamed through LDS in stages (t addresses the stage's rows;
+// t.n = keys left from the stage's first one).  `first`: the stage opens the sequence (negm is zero and the row's
+// reference is taken from the stage's first block); otherwise the running reference in negm is carried on.  The
+// last block is masked when t.n < 32 NB.
+template <int NB>
+__device__ __forceinline__ void att_stage_fixed(const AttnTile &t, const int (&cs)[4], bool first,
+                                                const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm, float (&l)[2])
+{
+    u32x4 kf[4];
+    f32x16 sbuf[2];
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) kf[sl] = att_read_k(t, cs, 0, sl);
+    sbuf[0] = att_mfma(kf[0], qf[0], negm);
+    sbuf[0] = att_mfma(kf[1], qf[1], sbuf[0]);
+    sbuf[0] = att_mfma(kf[2], qf[2], sbuf[0]);
+    sbuf[0] = att_mfma(kf[3], qf[3], sbuf[0]);
+    if constexpr (NB > 1) {
+#pragma unroll
+        for (int sl = 0; sl < 4; sl++) kf[sl] = att_read_k(t, cs, 1, sl);
+    }
+    if (first) {                                     // wave-uniform
+        if (NB == 1 && t.n < 32) {                   // a lone, partial block: its missing keys must not set the reference
+            const int lim = t.n - 4 * t.lg;
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                if (8 * (e >> 2) + (e & 3) >= lim) sbuf[0][e] = -INFINITY;
+        }
+        float m = att_max16(sbuf[0]);
+        m = fmaxf(m, __shfl_xor(m, 32, WAVE));       // key 0 always exists: m is finite
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            sbuf[0][e] -= m;
+            negm[e] = -m;
+        }
+    }
+    const bool partial = t.n < 32 * NB;              // wave-uniform
+    static_for<NB>([&](auto kbc) {
+        constexpr int kb = decltype(kbc)::value;
+        constexpr bool NEXT = kb + 1 < NB, NEXT2 = kb + 2 < NB;
+        if constexpr (kb == NB - 1) {
+            if (partial) att_step<NEXT, NEXT2, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            else att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+        } else {
+            att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+        }
+    });
 }
 
 #undef VT_PIN
@@ -509,27 +477,76 @@ __global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_ke
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Streaming variant (any n): K/V stages of 128 keys double buffered in LDS, workgroup = 128 query rows.
-__global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_kernel(
+// Longer key sequences (512 px models, spatially reduced PVT stages): a workgroup of four waves takes 128 query
+// rows of one (sample, head), a wave 32 of them, and the keys and values pass through LDS in stages of 128 (four
+// blocks of the tile pipeline above), double buffered: the direct loads of stage s+1 are issued before stage s is
+// multiplied and waited for after it.  Two workgroups share a compute unit, out of step with each other (with
+// eight waves and 256 rows per workgroup the per-stage barrier makes every SIMD wait for its slower wave:
+// measured 7 % slower).  K and V rows are laid out as in the resident kernel (V transposed by the LDS read).
+constexpr int ASK = 128;                            // keys per stage
+constexpr int ASBUF = 2 * ASK * 128;                // one stage: K rows, then V rows
+
+__global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_stream_kernel(
     const bf16_t *__restrict__ q, int64_t q_rs, int64_t q_hs, const bf16_t *__restrict__ k,
     const bf16_t *__restrict__ v, int64_t kv_bs, int64_t kv_ts, int64_t kv_hs, const int64_t *__restrict__ offsets,
-    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, int qchunks, float scale)
+    bf16_t *__restrict__ out, int64_t o_rs, int64_t o_hs, int n, int qchunks, float scale, int items, int h)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
-    const int b = blockIdx.x / qchunks, qc = blockIdx.x % qchunks;
-    const int head = blockIdx.y;
+    extern __shared__ __attribute__((aligned(128))) unsigned char smem[];
+    // Workgroups are dealt to the eight XCDs in turn (id % 8).  The query chunks of one (sample, head) all stream the
+    // same keys and values: they are given ids that land on one XCD, one after the other, so that its L2 fetches
+    // them from memory once.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int item = (slot / qchunks) * 8 + xcd, qc = slot % qchunks;
+    if (item >= items) return;
+    const int b = item / h, head = item - b * h;
     const int64_t row0 = offsets[b];
     const int Lb = (int)(offsets[b + 1] - row0);
     if (qc * AQ >= Lb) return;
 
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lg = lane >> 5;
     const int qrow = qc * AQ + wid * 32 + lr;
     const bool wave_live = qc * AQ + wid * 32 < Lb;
     const bool row_live = qrow < Lb;
+    const float c = scale * 1.44269504088896340736f;
+    const int64_t row_bytes = kv_ts * 2;
+    const void *kbase = uniform_ptr(k + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
+    const void *vbase = uniform_ptr(v + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
+    const int nstage = (n + ASK - 1) / ASK;
 
-    // Q fragments (B operand of S^T): bytes [32 s + 16 g, +16) of the query row
+    // stage st into buffer st & 1: wave-load j covers rows 8j .. 8j+7 of K (j < 16) or of V; this wave issues the
+    // loads j = wid, wid + 4, ..., whose lane offsets and LDS addresses are worked out once.  Issued from assembly so
+    // that the compiler does not wait for them before the LDS reads of the stage being multiplied.
+    constexpr int NLD = 2 * (ASK / 8) / (AQ / 32);       // loads per wave and stage
+    uint32_t ld_off[NLD], ld_row[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+        const int j = wid + i * (AQ / 32);
+        const bool is_v = j >= ASK / 8;
+        const int r = (is_v ? j - ASK / 8 : j) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ (is_v ? 2 * (r & 3) : (r >> 1) & 7);
+        ld_row[i] = (uint32_t)r;
+        ld_off[i] = (uint32_t)(r * row_bytes + chunk * 16);
+    }
+    auto issue = [&](int st) {
+        const uint32_t lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(smem + (st & 1) * ASBUF + wid * 1024));
+        const uint32_t stage_off = (uint32_t)(st * ASK * row_bytes);
+        const bool whole = (st + 1) * ASK <= n;          // wave-uniform: no row of the stage lies past the keys
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            const bool is_v = wid + i * (AQ / 32) >= ASK / 8;      // the same for every wave: AQ / 32 divides ASK / 8
+            uint32_t off = ld_off[i] + stage_off;
+            if (!whole) {
+                const int key = st * ASK + (int)ld_row[i];
+                if (key >= n) off -= (uint32_t)((key - (n - 1)) * row_bytes);        // repeat the last key
+            }
+            dma16(is_v ? vbase : kbase, off, lds + i * (AQ / 32) * 1024);
+        }
+    };
+    issue(0);
+
+    // Q fragments (second operand of S^T): bytes [32 s + 16 g, +16) of the query row, times scale * log2(e)
     u32x4 qf[4];
     {
         const unsigned char *qp =
@@ -539,85 +556,42 @@ __global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_kernel(
             const u32x4 z = {0u, 0u, 0u, 0u};
             qf[s] = row_live ? *reinterpret_cast<const u32x4 *>(qp + s * 32) : z;
         }
+#pragma unroll
+        for (int s = 0; s < 4; s++) qf[s] = att_scale_frag(qf[s], c);
     }
-
-    const unsigned char *kbase = reinterpret_cast<const unsigned char *>(k + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
-    const unsigned char *vbase = reinterpret_cast<const unsigned char *>(v + (int64_t)b * kv_bs + (int64_t)head * kv_hs);
-    const int64_t row_bytes = kv_ts * 2;
-    const int nstage = (n + AK - 1) / AK;
-
-    // K direct loads: wave-load j = wid*4 + i covers keys 8j..8j+7 of the stage
-    auto issue_k = [&](int st) {
-        unsigned char *dst = smem + (st & 1) * ABUF + wid * 4 * 1024;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int r = (wid * 4 + i) * 8 + (lane >> 3);
-            const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-            int key = st * AK + r;
-            key = key < n ? key : n - 1;
-            VT_GLOBAL_TO_LDS(kbase + key * row_bytes + chunk * 16, dst + i * 1024);
-        }
-    };
-    // V: thread -> (key, 16-byte chunk of d); registers now, transposed LDS writes later
-    u32x4 vreg[4];
-    auto load_v = [&](int st) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int idx = tid + 256 * i;
-            int key = st * AK + (idx >> 3);
-            key = key < n ? key : n - 1;
-            vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + key * row_bytes + (idx & 7) * 16);
-        }
-    };
-    auto store_v = [&](int st) {
-        unsigned char *vt = smem + (st & 1) * ABUF + AK * 128;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int idx = tid + 256 * i;
-            const int kr = idx >> 3, ch = idx & 7;
-            const int kpos = kr ^ (8 * ((ch >> 1) & 3));       // (d >> 4) & 3 with d = 8*ch + e
-            const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint16_t h16 = (uint16_t)(e & 1 ? w[e >> 1] >> 16 : w[e >> 1] & 0xffffu);
-                *reinterpret_cast<uint16_t *>(vt + (ch * 8 + e) * AVP + kpos * 2) = h16;
-            }
-        }
-    };
-
-    f32x16 o[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) o[i][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-    const float c = scale * 1.44269504088896340736f;
-
-    // fragment addressing
     const int sw = (lr >> 1) & 7;
     int cs[4];
 #pragma unroll
     for (int s = 0; s < 4; s++) cs[s] = ((2 * s + lg) ^ sw) * 16;
-    issue_k(0);
-    load_v(0);
-    store_v(0);
-    for (int st = 0; st < nstage; st++) {
-        wait_vmcnt<0>();                 // K of this stage (and nothing else is outstanding)
-        __syncthreads();                 // K and V^T of stage st visible; the other buffer is free
-        if (st + 1 < nstage) {
-            issue_k(st + 1);
-            load_v(st + 1);
-        }
-        if (wave_live) {
-            const int key0 = st * AK;
-            const unsigned char *ks = smem + (st & 1) * ABUF;
-            if (key0 + AK <= n) attn_stage<true>(ks, ks + AK * 128, AVP, 0, key0, n, lr, lg, cs, qf, o, m_run, l_run, c);
-            else attn_stage<false>(ks, ks + AK * 128, AVP, 0, key0, n, lr, lg, cs, qf, o, m_run, l_run, c);
-        }
-        if (st + 1 < nstage) store_v(st + 1);    // buffer (st+1)&1 was last read in iteration st-1
-    }
 
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 o[2] = {zero, zero}, negm = zero;
+    float l[2] = {0.f, 0.f};
+    const int nfull = n / ASK;                        // stages of four whole blocks; then at most one shorter stage
+    auto stage_tile = [&](int st) {
+        const unsigned char *buf = smem + (st & 1) * ASBUF;
+        return AttnTile{buf + lr * 128, att_v_lane(buf + ASK * 128, lane), n - st * ASK, lg};
+    };
+    for (int st = 0; st < nfull; st++) {
+        wait_vmcnt<0>();                 // this wave's loads of stage st (nothing younger is in flight)
+        __syncthreads();                 // stage st is complete; the other buffer was last read in iteration st-1
+        if (st + 1 < nstage) issue(st + 1);
+        if (wave_live) att_stage_fixed<4>(stage_tile(st), cs, st == 0, qf, o, negm, l);
+    }
+    if (nfull < nstage) {                // the last, shorter stage: 1 .. 3 blocks (its own code, outside the loop)
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (wave_live) {
+            const AttnTile tile = stage_tile(nfull);
+            switch ((tile.n + 31) / 32) {
+            case 3: att_stage_fixed<3>(tile, cs, nfull == 0, qf, o, negm, l); break;
+            case 2: att_stage_fixed<2>(tile, cs, nfull == 0, qf, o, negm, l); break;
+            default: att_stage_fixed<1>(tile, cs, nfull == 0, qf, o, negm, l); break;
+            }
+        }
+    }
     if (!wave_live) return;
+    const float l_run = l[0] + l[1];
     const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
     if (row_live) attn_store(out + (row0 + qrow) * o_rs + (int64_t)head * o_hs, o, l_tot, lg);
 }
@@ -655,13 +629,14 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
         }
 #undef VT_ATT_PIPE
     }
-    const size_t lds = 2 * (size_t)ABUF;
+    const size_t lds = 2 * (size_t)ASBUF;
     const int qchunks = (int)ceil_div(max_rows, AQ);
-    auto kern = sparse_attention_bf16_d64_kernel;
+    auto kern = sparse_attention_bf16_d64_stream_kernel;
     VT_RESERVE_LDS(kern, lds, "sparse_attention");
-    dim3 grid((unsigned)((int64_t)B * qchunks), (unsigned)h), block(256);
+    const int items = B * h;
+    dim3 grid((unsigned)(ceil_div(items, 8) * 8 * qchunks)), block(AQ * 2);
     kern<<<grid, block, lds, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v, kv_bs, kv_ts,
-                                   kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, qchunks, scale);
+                                   kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, qchunks, scale, items, h);
     return check_launch("sparse_attention");
 }
 
