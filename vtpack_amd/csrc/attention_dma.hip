@@ -409,19 +409,30 @@ __global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_ke
     // Rows past the last key repeat it (their scores are masked).  Issued from assembly: the compiler would
     // otherwise wait for every direct load in flight before any later read of LDS, i.e. put the prefetch in front
     // of the arithmetic it is meant to overlap.
+    // Lane constants of a wave-load: row (lane / 8) of its eight rows, chunk position lane % 8; the chunk fetched for
+    // a position depends on the row through the swizzle (K: on (row / 2) % 8, i.e. on the parity of j as well; V: on
+    // row % 4 only).
+    const int lrow = lane >> 3, lchunk = lane & 7;
+    const uint32_t lrow_off = (uint32_t)(lrow * row_bytes);
+    const uint32_t koff[2] = {lrow_off + (uint32_t)((lchunk ^ (lrow >> 1)) * 16),
+                              lrow_off + (uint32_t)((lchunk ^ (4 + (lrow >> 1))) * 16)};
+    const uint32_t voff = lrow_off + (uint32_t)((lchunk ^ (2 * (lrow & 3))) * 16);
     auto stage_issue = [&](const Item &im, unsigned char *buf, int w0, int nw) {
-        const unsigned char *kbase =
-            reinterpret_cast<const unsigned char *>(k + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
-        const unsigned char *vbase =
-            reinterpret_cast<const unsigned char *>(v + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
-        const int lf = fresh(lane);
+        const void *kbase = uniform_ptr(k + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
+        const void *vbase = uniform_ptr(v + (int64_t)im.b * kv_bs + (int64_t)im.head * kv_hs);
+        const uint32_t lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)buf);
         for (int j = w0; j < 2 * (npad / 8); j += nw) {
             const bool is_v = j >= npad / 8;
-            const int r = (is_v ? j - npad / 8 : j) * 8 + (lf >> 3);
-            const int chunk = (lf & 7) ^ (is_v ? 2 * (r & 3) : (r >> 1) & 7);
-            const int key = r < n ? r : n - 1;
-            dma16(uniform_ptr(is_v ? vbase : kbase), (uint32_t)(key * row_bytes + chunk * 16),
-                  (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(buf + j * 1024)));
+            const int jj = is_v ? j - npad / 8 : j;
+            uint32_t off;
+            if (jj * 8 + 8 <= n) {             // wave-uniform: all eight rows exist
+                off = (is_v ? voff : koff[jj & 1]) + (uint32_t)(jj * 8 * row_bytes);
+            } else {
+                const int r = jj * 8 + lrow;
+                const int chunk = lchunk ^ (is_v ? 2 * (r & 3) : (r >> 1) & 7);
+                off = (uint32_t)((r < n ? r : n - 1) * row_bytes + chunk * 16);
+            }
+            dma16(is_v ? vbase : kbase, off, lds + j * 1024);
         }
     };
 
@@ -472,7 +483,10 @@ __global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_ke
         if (wid >= NW / 2) wait_vmcnt<0>();
 #pragma unroll
         for (int s = 0; s < 4; s++) qf[s] = qn[s];
-        __syncthreads();      // the next item's buffer is complete; this item's buffer is free
+        // The next item's buffer is complete (its loaders have waited) and this item's buffer is free (its fragments
+        // are in registers or consumed).  A plain barrier: the fence of __syncthreads() would make every wave wait
+        // for its output stores as well.
+        block_barrier();
     }
 }
 
