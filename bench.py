@@ -95,7 +95,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         if dt == "bf16" and tag[3] == 64:
             if tag[4] <= 288:
                 return f"sparse_attention_bf16_d64_pipelined_kernel<{-(-tag[4] // 32)}>"
-            return "sparse_attention_bf16_d64_kernel"
+            return "sparse_attention_bf16_d64_stream_kernel"
         return f"sparse_attention_kernel<{T}, {tag[3]}>"
     if name == "vtdge_router":
         return f"router_kernel<{T}, 4, {gs(tag[1])}, false>"     # region size 4 in every model of these workloads
