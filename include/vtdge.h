@@ -173,6 +173,31 @@ int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void
                            const void *residual, int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev,
                            int64_t rows, int N, int K, int act, int dtype, void *stream);
 
+/* LayerNorm folded into the Linear that consumes it: out = act(LayerNorm(A) W^T + bias) computed from the raw rows
+ * of A, so that nn.LayerNorm followed by nn.Linear (norm1 -> kv and norm2 -> fc1,
+ * vtpack/models/dge/deit_dge.py:127-128 with :73 and :38-44) costs no pass over the rows of its own:
+ *     LayerNorm(a) W^T + bias = rstd * (a W'^T - mean * colsum(W') + sigma * b'),
+ *     W' = W * ln_weight (rounded to the storage type),  b' = bias + W ln_bias,  sigma = 1 / rstd = sqrt(var + eps).
+ *   vtdge_layernorm_stats   records [rows, 16] bf16 (32 bytes a row): mean and sigma of every row of x [rows, C],
+ *                           each split into bf16 parts in the operand order of the matrix instruction (two-pass
+ *                           fp32 statistics, as vtdge_layernorm).  Other kernels that produce the rows can write
+ *                           the same records (see vtdge_decompress_router, vtdge_linear_stats).
+ *   vtdge_layernorm_fold    once per weight: W_folded [N, K] = W', col_records [N, 16] bf16 = -colsum(W') and b'
+ *                           in the matching order.  bias is nullable.
+ *   vtdge_linear_layernorm  the Linear: A [rows, K] raw rows with their row_records, W_folded (and optionally its
+ *                           packed copy from vtdge_linear_prepack), col_records.  Weight-stationary kernel only:
+ *                           bf16, K = 384, N a multiple of 384 up to 3072, rows >= 2048 (capacity; the live count
+ *                           may be anything), else VTDGE_ERR_UNSUPPORTED.
+ * Against vtdge_layernorm followed by vtdge_linear the result differs by the rounding of W' instead of that of
+ * LayerNorm(a) to bf16: the same order of magnitude, not the same bits. */
+int vtdge_layernorm_stats(const void *x, void *records, const int64_t *rows_dev, int64_t rows, int C, float eps,
+                          int dtype, void *stream);
+int vtdge_layernorm_fold(const void *W, const void *bias, const void *ln_weight, const void *ln_bias, int N, int K,
+                         int dtype, void *W_folded, void *col_records, void *stream);
+int vtdge_linear_layernorm(const void *A, int64_t lda, const void *row_records, const void *W_folded,
+                           const void *packed, const void *col_records, void *out, int64_t ldo,
+                           const int64_t *rows_dev, int64_t rows, int N, int K, int act, int dtype, void *stream);
+
 /* Sparse attention of packed queries against each sample's full K/V:
  *   out[rows of sample i, head a] = softmax(scale * Q_i,a K_i,a^T) V_i,a
  * Replaces batched_sparse_attention_forward

@@ -73,6 +73,46 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
+// Statistics record of a row for the Linear that layer-normalises its input on the fly (linear_ws.hip, HAS_LN):
+// 16 bf16 values, the A-side operand of one 16-deep MFMA K step.  mean = m1 + m2 + m3 and sigma = sqrt(var + eps)
+// = s1 + s2 are split into bf16 parts; against the column record (-c1, -c2, -c1, -c3, -c2, -c1, b1, b1 | b2, 0, ...)
+// of a column with colsum c = c1 + c2 + c3 and bias b = b1 + b2 the K step yields -mean * c + sigma * b with all
+// partial products of weight 2^-24 and above (2^-16 for the bias term).  Both halves carry (s1, s2) so that every
+// lane of the consumer finds sigma in its own half.
+//   lo = (m1, m1, m2, m1, m2, m3, s1, s2)   hi = (s1, s2, 0, 0, 0, 0, 0, 0)
+__device__ __forceinline__ void split_bf16x3(float v, uint32_t &p1, uint32_t &p2, uint32_t &p3)
+{
+    p1 = f32_to_bf16(v);
+    const float r1 = v - bf16_to_f32((bf16_t)p1);
+    p2 = f32_to_bf16(r1);
+    p3 = f32_to_bf16(r1 - bf16_to_f32((bf16_t)p2));
+}
+__device__ __forceinline__ void ln_record(float mean, float sigma, u32x4 &lo, u32x4 &hi)
+{
+    uint32_t m1, m2, m3, s1, s2, s3;
+    split_bf16x3(mean, m1, m2, m3);
+    split_bf16x3(sigma, s1, s2, s3);
+    lo.x = m1 | (m1 << 16);
+    lo.y = m2 | (m1 << 16);
+    lo.z = m2 | (m3 << 16);
+    lo.w = s1 | (s2 << 16);
+    hi.x = s1 | (s2 << 16);
+    hi.y = hi.z = hi.w = 0u;
+}
+// the matching record of an output column: colsum of the folded weights and the folded bias
+__device__ __forceinline__ void ln_column_record(float colsum, float b, u32x4 &lo, u32x4 &hi)
+{
+    uint32_t c1, c2, c3, b1, b2, b3;
+    split_bf16x3(-colsum, c1, c2, c3);
+    split_bf16x3(b, b1, b2, b3);
+    lo.x = c1 | (c2 << 16);
+    lo.y = c1 | (c3 << 16);
+    lo.z = c2 | (c1 << 16);
+    lo.w = b1 | (b1 << 16);
+    hi.x = b2;
+    hi.y = hi.z = hi.w = 0u;
+}
+
 // Storage-type traits: a 16-byte vector of T holds VEC elements.
 template <typename T> struct Elem;
 template <> struct Elem<float> {

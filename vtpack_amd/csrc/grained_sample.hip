@@ -992,6 +992,64 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
     }
 }
 
+// The statistics half of layernorm_kernel: per row the 32-byte record (mean and sqrt(var + eps), see ln_record)
+// that a Linear with a folded LayerNorm takes next to the raw rows.  Same two-pass arithmetic and reduction tree.
+template <int NIT, int GS>
+__global__ __launch_bounds__(256) void layernorm_stats_kernel(const bf16_t *__restrict__ x, u32x4 *__restrict__ rec,
+                                                               const int64_t *__restrict__ rows_dev, int64_t rows,
+                                                               int C, float eps)
+{
+    constexpr int VEC = 8;
+    const int lane = threadIdx.x & (GS - 1);
+    const int64_t live = live_rows(rows_dev, rows);
+    const int64_t row0 =
+        (((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS) * LN_RPW;
+    if (row0 >= live) return;
+    const int nvec = C / VEC;
+    u32x4 raw[LN_RPW][NIT];
+#pragma unroll
+    for (int r = 0; r < LN_RPW; r++)
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int v = it * WAVE + lane;
+            if (v < nvec && row0 + r < live)
+                raw[r][it] = *reinterpret_cast<const u32x4 *>(x + (row0 + r) * (int64_t)C + v * VEC);
+        }
+#pragma unroll
+    for (int r = 0; r < LN_RPW; r++) {
+        if (row0 + r >= live) break;
+        float vals[NIT][VEC];
+        float s = 0.f;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            if (it * WAVE + lane < nvec) {
+                Elem<bf16_t>::unpack(raw[r][it], vals[it]);
+#pragma unroll
+                for (int c = 0; c < VEC; c++) s += vals[it][c];
+            }
+        }
+        const float mean = group_sum<GS>(s) / (float)C;
+        float q = 0.f;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            if (it * WAVE + lane < nvec) {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    const float dlt = vals[it][c] - mean;
+                    q += dlt * dlt;
+                }
+            }
+        }
+        const float sigma = sqrtf(group_sum<GS>(q) / (float)C + eps);
+        if (lane == 0) {
+            u32x4 lo, hi;
+            ln_record(mean, sigma, lo, hi);
+            rec[(row0 + r) * 2] = lo;
+            rec[(row0 + r) * 2 + 1] = hi;
+        }
+    }
+}
+
 // ------------------------------------------------------------- host side
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -1300,4 +1358,26 @@ extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bi
 #undef VT_GROUP
 #undef VT_LAUNCH
     return check_launch("layernorm");
+}
+
+extern "C" int vtdge_layernorm_stats(const void *x, void *records, const int64_t *rows_dev, int64_t rows, int C,
+                                     float eps, int dtype, void *stream)
+{
+    VT_REQUIRE(x && records, VTDGE_ERR_ARG, "layernorm_stats: NULL operand");
+    VT_REQUIRE(rows >= 0, VTDGE_ERR_ARG, "layernorm_stats: negative rows");
+    VT_REQUIRE(dtype == VTDGE_BF16, VTDGE_ERR_UNSUPPORTED, "layernorm_stats: records exist for bf16 rows only");
+    if (int rc = check_channels(C, dtype, "layernorm_stats")) return rc;
+    VT_REQUIRE(C / 8 <= WAVE * MAX_IT, VTDGE_ERR_UNSUPPORTED, "layernorm_stats: C=%d exceeds %d", C, WAVE * MAX_IT * 8);
+    VT_REQUIRE(aligned16(x) && aligned16(records), VTDGE_ERR_ARG, "layernorm_stats: operands must be 16-byte aligned");
+    if (rows == 0) return VTDGE_OK;
+    const int gs = group_size(C / 8);
+    dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * LN_RPW * (WAVE / gs))), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    const int nit = (int)ceil_div(C / 8, WAVE);
+#define VT_LAUNCH(NIT, GS) \
+    layernorm_stats_kernel<NIT, GS><<<grid, block, 0, st>>>((const bf16_t *)x, (u32x4 *)records, rows_dev, rows, C, eps)
+    if (gs == 64) { if (nit == 1) VT_LAUNCH(1, 64); else if (nit == 2) VT_LAUNCH(2, 64); else VT_LAUNCH(3, 64); }
+    else if (gs == 32) VT_LAUNCH(1, 32); else if (gs == 16) VT_LAUNCH(1, 16); else VT_LAUNCH(1, 8);
+#undef VT_LAUNCH
+    return check_launch("layernorm_stats");
 }

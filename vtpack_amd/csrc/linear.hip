@@ -192,6 +192,10 @@ int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, 
                      int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
                      hipStream_t st);
 
+int launch_linear_ws_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
+                        const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
+                        hipStream_t st);
+
 // K-split weight-stationary variant for bf16, K = 1536, narrow N (linear_ks.hip)
 bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
@@ -259,6 +263,70 @@ extern "C" int vtdge_linear_prepack(const void *W, int N, int K, int dtype, void
     linear_prepack_kernel<<<(unsigned)ceil_div(units, 256), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t *)W, (u32x4 *)packed, N, K, layout);
     return check_launch("linear_prepack");
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// LayerNorm folded into the Linear that follows it:  LayerNorm(a) W^T + bias = rstd * (a W'^T - mean * colsum(W')
+// + sigma * b')  with W' = W * gamma (rounded to bf16, the value the MFMAs multiply by) and b' = bias + W beta.
+// One wave per output column writes the row of W' and the column's record (see ln_column_record).
+__global__ __launch_bounds__(256) void layernorm_fold_kernel(const bf16_t *__restrict__ W, const bf16_t *__restrict__ bias,
+                                                              const bf16_t *__restrict__ gamma,
+                                                              const bf16_t *__restrict__ beta, bf16_t *__restrict__ Wf,
+                                                              u32x4 *__restrict__ colrec, int N, int K)
+{
+    const int col = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (col >= N) return;
+    float cs = 0.f, wb = 0.f;
+    for (int k = lane; k < K; k += 64) {
+        const float w = bf16_to_f32(W[(int64_t)col * K + k]);
+        const bf16_t f = f32_to_bf16(w * bf16_to_f32(gamma[k]));
+        Wf[(int64_t)col * K + k] = f;
+        cs += bf16_to_f32(f);
+        wb += w * bf16_to_f32(beta[k]);
+    }
+    cs = wave_sum(cs);
+    wb = wave_sum(wb);
+    if (lane == 0) {
+        u32x4 lo, hi;
+        ln_column_record(cs, wb + (bias ? bf16_to_f32(bias[col]) : 0.f), lo, hi);
+        colrec[col * 2] = lo;
+        colrec[col * 2 + 1] = hi;
+    }
+}
+
+extern "C" int vtdge_layernorm_fold(const void *W, const void *bias, const void *ln_weight, const void *ln_bias, int N,
+                                    int K, int dtype, void *W_folded, void *col_records, void *stream)
+{
+    VT_REQUIRE(W && ln_weight && ln_bias && W_folded && col_records, VTDGE_ERR_ARG, "layernorm_fold: NULL operand");
+    VT_REQUIRE(N > 0 && K > 0, VTDGE_ERR_ARG, "layernorm_fold: bad sizes N=%d K=%d", N, K);
+    VT_REQUIRE(dtype == VTDGE_BF16, VTDGE_ERR_UNSUPPORTED, "layernorm_fold: built for bf16 weights only");
+    VT_REQUIRE(((uintptr_t)col_records & 15) == 0, VTDGE_ERR_ARG, "layernorm_fold: records must be 16-byte aligned");
+    layernorm_fold_kernel<<<(unsigned)ceil_div(N, 4), 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)ln_weight, (const bf16_t *)ln_bias, (bf16_t *)W_folded,
+        (u32x4 *)col_records, N, K);
+    return check_launch("layernorm_fold");
+}
+
+extern "C" int vtdge_linear_layernorm(const void *A, int64_t lda, const void *row_records, const void *W_folded,
+                                      const void *packed, const void *col_records, void *out, int64_t ldo,
+                                      const int64_t *rows_dev, int64_t rows, int N, int K, int act, int dtype,
+                                      void *stream)
+{
+    VT_REQUIRE(A && row_records && W_folded && col_records && out, VTDGE_ERR_ARG, "linear_layernorm: NULL operand");
+    VT_REQUIRE(act == VTDGE_ACT_NONE || act == VTDGE_ACT_GELU, VTDGE_ERR_ARG, "linear_layernorm: unknown activation %d",
+               act);
+    VT_REQUIRE(rows >= 0 && N > 0 && K > 0, VTDGE_ERR_ARG, "linear_layernorm: bad sizes rows=%lld N=%d K=%d",
+               (long long)rows, N, K);
+    VT_REQUIRE(lda >= K && ldo >= N, VTDGE_ERR_ARG, "linear_layernorm: leading dim too small");
+    VT_REQUIRE((((uintptr_t)A | (uintptr_t)W_folded | (uintptr_t)packed | (uintptr_t)row_records |
+                 (uintptr_t)col_records) & 15) == 0,
+               VTDGE_ERR_ARG, "linear_layernorm: operands must be 16-byte aligned");
+    VT_REQUIRE(dtype == VTDGE_BF16 && linear_ws_applicable(lda, 0, ldo, rows, N, K, 2, act, nullptr, nullptr, out),
+               VTDGE_ERR_UNSUPPORTED,
+               "linear_layernorm: built for bf16, K = 384, N a multiple of 384 (at most 3072) and 2048 rows or more "
+               "(rows=%lld N=%d K=%d dtype=%d)", (long long)rows, N, K, dtype);
+    return launch_linear_ws_ln(A, lda, row_records, W_folded, packed, col_records, out, ldo, rows_dev, rows, N, act,
+                               (hipStream_t)stream);
 }
 
 extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,

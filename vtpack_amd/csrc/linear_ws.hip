@@ -93,11 +93,21 @@ __device__ __forceinline__ void gelu_part3(EpiUnit &u)
     u.f1 = u.f1 * (u.x1 * u.q1 + 0.5f);
 }
 
-template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES>
+// HAS_LN: the rows of A are to be layer-normalised first, out = act(LayerNorm(A) W^T + bias), without a normalised
+// copy of A.  With gamma folded into W (W' = W * gamma, rounded to bf16) and b' = bias + W beta,
+//     LayerNorm(a) W^T + bias = rstd * (a W'^T - mean * colsum(W') + sigma * b'),   sigma = 1 / rstd,
+// so the tile loop multiplies the raw rows by W' and one more K step adds the two rank-one terms: its A-side
+// fragment is the row's 32-byte statistics record (mean and sigma, each split into bf16 parts so that the products
+// carry 24 and 16 significant bits; written by whoever produced the row, see ln_record in common.h), its W-side
+// fragment the column's record of -colsum(W') and b' in the matching order (`lnw`, two 16-byte halves per output
+// column).  The records of a tile arrive in LDS with the tile (one more direct load, issued by wave 0); the
+// epilogue multiplies by rstd = 1 / (sigma_1 + sigma_2).  A separate bias is not taken (it is part of b').
+template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES, bool HAS_LN = false>
 __global__ __launch_bounds__(256) void linear_ws_kernel(
     const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
     const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
-    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp)
+    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp,
+    const u32x4 *__restrict__ lnrec = nullptr, const u32x4 *__restrict__ lnw = nullptr)
 {
     constexpr int KB = KS * 32;                 // bytes of one operand row
     constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
@@ -123,6 +133,8 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     static_assert(KS % (FD + 1) == 0, "the fragment ring keeps its phase from tile to tile");
     static_assert(EARLY <= PA && 2 * NL <= KS, "prologue / direct loads inside the K loop");
     constexpr int OFF_R = DA * TILE;
+    constexpr int OFF_L = 6 * TILE;             // statistics records of the tiles in the A ring, 1 KB each
+    static_assert(!(HAS_LN && HAS_BIAS), "with HAS_LN the bias is part of the column records");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -164,6 +176,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     // read from the residual tile like fragments of A.  bf16 x 1 is exact, so the sum is (A W^T + bias) + residual,
     // each rounded once in fp32, as with separate additions.
     uint32_t wb[NB];
+    u32x4 wl[NB];         // HAS_LN: the column records, W-side fragments of the statistics K step
     u32x4 eye[2];
     {
         const u32x4 z = {0u, 0u, 0u, 0u};
@@ -171,6 +184,8 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         for (int j = 0; j < NB; j++) {
             wb[j] = 0u;
             if constexpr (HAS_BIAS) wb[j] = lg == 0 ? (uint32_t)bias[col0 + j * 32 + lr] : 0u;
+            wl[j] = z;
+            if constexpr (HAS_LN) wl[j] = lnw[(col0 + j * 32 + lr) * 2 + lg];
         }
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -229,7 +244,19 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         m = (m & ~(0xffull << sh)) | ((uint64_t)(v & 0xff) << sh);
     };
     auto after_mark = [&](uint64_t m, int k) -> int { return (issued - (int)((m >> ((k & 7) * 8)) & 0xff)) & 0xff; };
+    // the statistics records of tile k's 32 rows (lane i: half i % 2 of row i / 2), wave 0 only
+    auto rec_dma = [&](int k) {
+        int gm = tile_row0(k) + (lane >> 1);
+        gm = gm < M32 ? gm : M32 - 1;
+        dma16(lnrec, (uint32_t)gm * 32u + (lane & 1) * 16u, lds0 + OFF_L + (k % DA) * 1024);
+    };
     auto issue_a_all = [&](int k) {      // prologue only; inside the K loop the six loads are spread out
+        if constexpr (HAS_LN) {
+            if (w == 0) {
+                rec_dma(k);
+                issued += 1;
+            }
+        }
 #pragma unroll
         for (int ii = 0; ii < NL; ii++) {
             if (M32 >= 32) tile_dma(A, lda2, 0, va, tile_row0(k), ii, ii & 1, lds0 + (k % DA) * TILE);
@@ -326,6 +353,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     // ---- epilogue of one tile, in NU units.  Unit n = 4 * (2j + q) + e turns the accumulator pair
     // (8q + e, 8q + 4 + e) of block j into elements e and 4 + e of the lane's 8-column vector (j, q).
     uint32_t e_w[4];        // packed pairs of the current vector
+    float rs_prev = 1.0f;   // HAS_LN: rstd of the lane's row in the tile whose epilogue is due
     float h0, h1;           // elements of an even unit waiting for their odd neighbours
     EpiUnit un;
     auto epi_part1 = [&](auto pp_tag, int n) {
@@ -335,6 +363,10 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                                                   __float_as_uint(acc[PP][j][8 * q + 4 + e]), false, false);
         un.f0 = __uint_as_float(r[0]);
         un.f1 = __uint_as_float(r[1]);
+        if constexpr (HAS_LN) {
+            un.f0 *= rs_prev;
+            un.f1 *= rs_prev;
+        }
         if constexpr (ACT == VTDGE_ACT_GELU) gelu_part1(un);
     };
     auto epi_part2 = [&](int n) {
@@ -396,18 +428,24 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         const bool has_r = HAS_RES && k + PR < nt;
         const int w6 = w * NL;
         const uint32_t mask_a = has_a ? 0x3fu << w6 : 0u, mask_r = has_r ? 0x3fu << w6 : 0u;
+        // wave 0 also brings the statistics records of tile k+PA: in its last substep, between the residual's load
+        // and A's
+        const bool has_l = HAS_LN && has_a && w == 0;
         {
-            const int start = issued, n = (has_a ? 1 : 0) + (has_r ? 1 : 0);
+            const int start = issued, n = (has_a ? 1 : 0) + (has_r ? 1 : 0), x = has_l ? 1 : 0;
             const int st = EPI ? (w6 + 1) / 4 + 1 : 0;        // stores before the loads of substep 6w+5
             if (has_r) set_mark(marks_r, k + PR, start + (NL - 1) * n + 1 + st);
-            if (has_a) set_mark(marks_a, k + PA, start + NL * n + st);
-            issued = start + NL * n + (EPI ? NB * 2 : 0);
+            if (has_a) set_mark(marks_a, k + PA, start + NL * n + x + st);
+            issued = start + NL * n + x + (EPI ? NB * 2 : 0);
         }
         const uint32_t dst_a = lds0 + ((k + PA) % DA) * TILE, dst_r = lds0 + OFF_R + ((k + PR) % DR) * TILE;
         const uint32_t sa = (uint32_t)tile_row0(k + PA) * lda2, sr = (uint32_t)tile_row0(k + PR) * ldr2 + g * KB;
         auto step_dma = [&](int s) {      // s is a compile-time constant at every call
             if constexpr (HAS_RES) {
                 if ((mask_r >> s) & 1) dma16(res, sr + (s & 3) * 8 * ldr2 + (s >> 2) * 128 + vr[s & 1], dst_r + s * 1024);
+            }
+            if constexpr (HAS_LN) {
+                if (s == NL - 1 && has_l) rec_dma(k + PA);
             }
             if ((mask_a >> s) & 1) dma16(A, sa + (s & 3) * 8 * lda2 + (s >> 2) * 128 + va[s & 1], dst_a + s * 1024);
         };
@@ -419,6 +457,13 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         const unsigned char *an = smem + ((k + 1) % DA) * TILE;
         unsigned char *orow = nullptr;
         if constexpr (EPI) orow = out_row(k - 1);
+        u32x4 fl = {0u, 0u, 0u, 0u};
+        float rs_cur = 1.0f;
+        if constexpr (HAS_LN) {
+            fl = *reinterpret_cast<const u32x4 *>(smem + OFF_L + (k % DA) * 1024 + lr * 32 + lg * 16);
+            const uint32_t sg = lg ? fl.x : fl.w;      // (sigma_1, sigma_2) sits in both halves of the record
+            rs_cur = __builtin_amdgcn_rcpf(__uint_as_float(sg << 16) + __uint_as_float(sg & 0xffff0000u));
+        }
         // residual fragments: K steps 6w .. 6w+5 of the residual tile, through a ring of four registers sets
         u32x4 fr[4];
         auto read_fr = [&](int i) {            // i-th fragment in the order the MFMAs take them
@@ -463,6 +508,11 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+        if constexpr (HAS_LN) {
+#pragma unroll
+            for (int j = 0; j < NB; j++) mma_v_fresh(acc[PP][j], wl[j], fl);
+            rs_prev = rs_cur;       // for this tile's epilogue, which runs during the next step
         }
         if constexpr (HAS_BIAS) {
             const u32x4 ones = {fresh(lane) < 32 ? 0x3f80u : 0u, 0u, 0u, 0u};   // made here: no registers held
@@ -532,14 +582,15 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
            (((uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15) == 0;
 }
 
-template <int ACT, bool HB, bool HR>
+template <int ACT, bool HB, bool HR, bool LN = false>
 static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
-                 int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st)
+                 int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st,
+                 const void *lnrec = nullptr, const void *lnw = nullptr)
 {
     constexpr int KS = 24, NB = 3;
-    constexpr size_t lds = (size_t)6 * 32 * KS * 32;   // six 32-row tiles
+    constexpr size_t lds = (size_t)6 * 32 * KS * 32 + (LN ? 4 * 1024 : 0);   // six 32-row tiles (+ four tiles' records)
     static_assert(lds <= 160 * 1024, "LDS budget");
-    auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR>;
+    auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR, LN>;
     VT_RESERVE_LDS(kern, lds, "linear");
     const int groups = N / (4 * NB * 32);
     // one workgroup per CU; the P workgroups of a column group are spread over the 8 XCDs, and the workgroups
@@ -549,8 +600,21 @@ static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, cons
     if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
     dim3 grid((unsigned)(P * groups)), block(256);
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
-                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp);
+                                   ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp,
+                                   (const u32x4 *)lnrec, (const u32x4 *)lnw);
     return check_launch("linear");
+}
+
+// out = act(LayerNorm(A) W^T + bias) from the raw rows, their statistics records and the folded weights
+int launch_linear_ws_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
+                        const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
+                        hipStream_t st)
+{
+    if (act == VTDGE_ACT_GELU)
+        return go_ws<VTDGE_ACT_GELU, false, false, true>(A, lda, Wf, Wfp, nullptr, nullptr, 0, out, ldo, rows_dev, rows,
+                                                          N, st, lnrec, lnw);
+    return go_ws<VTDGE_ACT_NONE, false, false, true>(A, lda, Wf, Wfp, nullptr, nullptr, 0, out, ldo, rows_dev, rows, N,
+                                                      st, lnrec, lnw);
 }
 
 int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,

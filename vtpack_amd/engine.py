@@ -31,6 +31,10 @@ FUSE_ROUTER_NORM = False
 # packed row: `vtdge_decompress_router`): the next block's router kernel and its pass over x disappear, and with it
 # the first kernel of the routing chain, the longer of the two chains.  On by default (same bits as the two kernels).
 FUSE_NEXT_ROUTER = True
+# The two LayerNorms of a block folded into the Linears that consume them (norm1 -> kv, norm2 -> fc1): the Linear
+# takes the raw rows and a 32-byte statistics record per row, so no normalised copy of the tokens is written or read.
+# Taken where the weight-stationary kernel applies (bf16, 384 channels, 2048 rows or more, no spatial reduction).
+FOLD_NORMS = True
 
 
 def _side_stream(device, slot=0):
@@ -52,6 +56,13 @@ def prepare(model):
             mod._vtdge_khwc = None
         if isinstance(mod, torch.nn.Linear) and mod.weight.is_cuda and mod.weight.dtype == torch.bfloat16:
             ops.packed_weight(mod.weight)
+        # a block's LayerNorms folded into the Linears behind them (see FOLD_NORMS)
+        if FOLD_NORMS and all(hasattr(mod, name) for name in ("norm1", "norm2", "attn", "mlp")):
+            for norm, lin in ((mod.norm1, getattr(mod.attn, "kv", None)), (mod.norm2, getattr(mod.mlp, "fc1", None))):
+                w = getattr(lin, "weight", None)
+                if (w is not None and w.is_cuda and w.dtype == torch.bfloat16 and w.shape[1] == 384
+                        and w.shape[0] % 384 == 0 and w.shape[0] <= 3072):
+                    ops.folded_weight(w, lin.bias, norm.weight, norm.bias)
     return model
 
 
@@ -123,11 +134,20 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
     # key/value chain (second stream)
     if overlap:
         side.wait_stream(main)
+    fold1 = (FOLD_NORMS and x_ln is None and getattr(attn, "sr_ratio", 1) <= 1
+             and ops.fits_linear_layernorm(x, attn.kv.weight))
     with torch.cuda.stream(side):
-        if x_ln is None:
-            x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
-        kv_src = _key_value_source(attn, x_ln, H, W, extra)
-        kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)                 # [B, n, 2C] = [B, n, 2, h, d]
+        if fold1:
+            rec1 = carry.get("x_stats")
+            if rec1 is None:
+                rec1 = ops.layernorm_stats(x, n1.eps)
+            kv_src = x
+            kv = ops.linear_layernorm(x, rec1, attn.kv.weight, attn.kv.bias, n1.weight, n1.bias)
+        else:
+            if x_ln is None:
+                x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
+            kv_src = _key_value_source(attn, x_ln, H, W, extra)
+            kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)             # [B, n, 2C] = [B, n, 2, h, d]
 
     # routing chain (caller's stream)
     if routed is not None:
@@ -147,12 +167,18 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
     if overlap:
         main.wait_stream(side)
         for t in (x_ln, kv_src, kv):
-            t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
+            if t is not None:
+                t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
     q1 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev)
 
-    q1_ln = ops.layernorm(q1, n2.weight, n2.bias, n2.eps, rows_dev=rows_dev)
-    hid = ops.linear(q1_ln, mlp.fc1.weight, mlp.fc1.bias, act="gelu", rows_dev=rows_dev)
+    if FOLD_NORMS and ops.fits_linear_layernorm(q1, mlp.fc1.weight):
+        rec2 = ops.layernorm_stats(q1, n2.eps, rows_dev=rows_dev)
+        hid = ops.linear_layernorm(q1, rec2, mlp.fc1.weight, mlp.fc1.bias, n2.weight, n2.bias, act="gelu",
+                                   rows_dev=rows_dev)
+    else:
+        q1_ln = ops.layernorm(q1, n2.weight, n2.bias, n2.eps, rows_dev=rows_dev)
+        hid = ops.linear(q1_ln, mlp.fc1.weight, mlp.fc1.bias, act="gelu", rows_dev=rows_dev)
     q2 = ops.linear(hid, mlp.fc2.weight, mlp.fc2.bias, residual=q1, rows_dev=rows_dev)
 
     handed = {}

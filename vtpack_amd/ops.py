@@ -256,6 +256,8 @@ def invalidate_packed(obj=None):
     for t in tensors:
         if getattr(t, "_vtdge_packed", None) is not None:
             t._vtdge_packed = None
+        if getattr(t, "_vtdge_folded", None) is not None:
+            t._vtdge_folded = None
 
 
 def packed_weight(weight):
@@ -315,6 +317,91 @@ def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=N
          (r2.stride(0) if rows > 1 else N) if r2 is not None else 0, ptr(o2), o2.stride(0) if rows > 1 else N,
          ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr(),
          tag=("linear", act, bias is not None, residual is not None, rows, N, K, rows_dev is not None))
+    return out
+
+
+# ------------------------------------------------------------------ LayerNorm folded into the Linear behind it
+def fits_linear_layernorm(a, weight):
+    """Whether `linear_layernorm` has a kernel for these operands (bf16, rows of 384, 2048 rows or more, an output
+    width that is a multiple of 384 up to 3072)."""
+    K = a.shape[-1]
+    rows = a.numel() // max(K, 1)
+    return (a.is_cuda and a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and K == 384
+            and weight.dim() == 2 and weight.shape[1] == K and weight.shape[0] % 384 == 0 and weight.shape[0] <= 3072
+            and rows >= 2048 and a.stride(-1) == 1)
+
+
+def layernorm_stats(x, eps=1e-6, rows_dev=None, out=None):
+    """The statistics records [rows, 16] bf16 of the rows of x [..., C] (bf16): what `linear_layernorm` takes next to
+    the raw rows instead of a normalised copy."""
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("layernorm_stats: records exist for bfloat16 rows only")
+    x = _contig(x)
+    C = x.shape[-1]
+    rows = x.numel() // C
+    if out is None:
+        out = torch.empty((rows, 16), dtype=torch.bfloat16, device=x.device)
+    elif out.shape != (rows, 16) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError(f"records must be a contiguous bfloat16 tensor of shape ({rows}, 16)")
+    call("vtdge_layernorm_stats", ptr(x), ptr(out), ptr(rows_dev), rows, C, float(eps), dtype_code(x), stream_ptr(),
+         tag=("layernorm_stats", rows, C))
+    return out
+
+
+def folded_weight(weight, bias, ln_weight, ln_bias):
+    """-> (W', column records, packed copy of W' or None) for `linear_layernorm`: the Linear's weight with the
+    LayerNorm's scale folded in, and per output column the colsum of W' and bias + W @ ln_bias.  Made once per set of
+    tensors and versions and kept on the weight tensor; `invalidate_packed` drops it like the packed copies."""
+    parts = (weight, bias, ln_weight, ln_bias)
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype, t.device) if t is not None else None
+                for t in parts) + (_pack_epoch,)
+    cached = getattr(weight, "_vtdge_folded", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    N, K = weight.shape
+    _check_like(weight, bias=bias, ln_weight=ln_weight, ln_bias=ln_bias)
+    _check_vector("bias", bias, N)
+    _check_vector("ln_weight", ln_weight, K)
+    _check_vector("ln_bias", ln_bias, K)
+    lib = _lib.load()        # not through call(): no part of a timed step
+    wf = torch.empty_like(weight, memory_format=torch.contiguous_format)
+    rec = torch.empty((N, 16), dtype=torch.bfloat16, device=weight.device)
+    if lib.vtdge_layernorm_fold(ptr(_contig(weight.detach())), ptr(None if bias is None else _contig(bias.detach())),
+                                ptr(_contig(ln_weight.detach())), ptr(_contig(ln_bias.detach())), N, K,
+                                dtype_code(weight), ptr(wf), ptr(rec), stream_ptr()) != 0:
+        raise _lib.VtdgeError(lib.vtdge_last_error().decode("utf-8", "replace"))
+    value = (wf, rec, packed_weight(wf) if PACK_WEIGHTS else None)
+    try:
+        weight._vtdge_folded = (key, value)
+    except AttributeError:
+        pass
+    return value
+
+
+def linear_layernorm(a, records, weight, bias, ln_weight, ln_bias, act="none", rows_dev=None, out=None):
+    """out = act(LayerNorm(a) @ weight.T + bias) from the raw rows a [..., 384] and their statistics records (from
+    `layernorm_stats` or from the kernel that produced the rows): no normalised copy of `a` is written or read.
+    The LayerNorm's eps is the one the records were made with."""
+    _need_gpu(a, weight, bias, ln_weight, ln_bias, records)
+    _check_like(a, weight=weight, bias=bias, ln_weight=ln_weight, ln_bias=ln_bias, out=out)
+    if not fits_linear_layernorm(a, weight):
+        raise ValueError("linear_layernorm: no kernel for these operands (see fits_linear_layernorm)")
+    K = a.shape[-1]
+    a2 = a.reshape(-1, K)
+    rows = a2.shape[0]
+    if records.shape != (rows, 16) or records.dtype != torch.bfloat16 or not records.is_contiguous():
+        raise ValueError(f"records must be a contiguous bfloat16 tensor of shape ({rows}, 16)")
+    N = weight.shape[0]
+    wf, colrec, packed = folded_weight(weight, bias, ln_weight, ln_bias)
+    if out is None:
+        out = torch.empty(a.shape[:-1] + (N,), dtype=a.dtype, device=a.device)
+    elif out.numel() != rows * N or out.shape[-1] != N:
+        raise ValueError(f"out {tuple(out.shape)} does not hold {rows} rows of {N}")
+    o2 = out.view(-1, N)
+    call("vtdge_linear_layernorm", ptr(a2), a2.stride(0), ptr(records), ptr(wf), ptr(packed), ptr(colrec), ptr(o2),
+         o2.stride(0), ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a),
+         stream_ptr(), tag=("linear_layernorm", act, rows, N, K, rows_dev is not None))
     return out
 
 
