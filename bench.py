@@ -79,7 +79,12 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
+    if name == "vtdge_linear_layernorm":
+        return f"linear_ws_kernel<24, 3, {1 if tag[1] == 'gelu' else 0}, false, false, true>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
+    if name == "vtdge_layernorm_stats":
+        nv = tag[2] * esz // 16
+        return f"layernorm_stats_kernel<{min(3, -(-nv // 64)) if gs(tag[2]) == 64 else 1}, {gs(tag[2])}>"
     if name == "vtdge_compress":
         return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}, {3 if tag[3] * esz // 16 > 64 else 1}>"
     if name == "vtdge_decompress":
@@ -87,7 +92,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
     if name == "vtdge_decompress_layernorm":
         return f"decompress_ln_kernel<{T}, {b(tag[1])}, {gs(tag[2])}>"
     if name == "vtdge_decompress_router":
-        return f"decompress_route_kernel<{T}, {gs(tag[3])}, {b(tag[1])}>"
+        return f"decompress_route_kernel<{T}, {gs(tag[3])}, {b(tag[1])}, {b(tag[4])}>"
     if name == "vtdge_layernorm":
         nv = tag[3] * esz // 16                           # 16-byte vectors per row
         return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
@@ -130,6 +135,14 @@ def algorithmic_work(name, tag, esz, geo):
         M = L if packed else rows
         # operands once: A, W, the output and, when there is one, the residual
         return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn * (2 if has_res else 1)) * esz
+    if name == "vtdge_linear_layernorm":
+        _, _, rows, Nn, K, packed = tag
+        M = L if packed else rows
+        # raw rows, their 32-byte records, the folded weights and their records, the output
+        return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn) * esz + 32 * (M + Nn)
+    if name == "vtdge_layernorm_stats":
+        rows = L if tag[1] != B * N else tag[1]
+        return "hbm", rows * tag[2] * esz + 32.0 * rows
     if name == "vtdge_sparse_attention":
         # tag[4] = keys per sample; bytes: q in, out, every sample's K and V once
         return "mfma", 4.0 * L * tag[4] * C, (2 * L * C + 2 * B * tag[4] * C) * esz
@@ -140,7 +153,8 @@ def algorithmic_work(name, tag, esz, geo):
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + (2 if tag[2] else 1) * B * N * C * esz
     if name == "vtdge_decompress_router":
         # the scatter-back's bytes: routing the next block reads nothing more (gate indices in, logits out: KBs)
-        return "hbm", (2 if tag[1] else 1) * L * C * esz + 2 * B * N * C * esz + 16 * B * geo["regions"]
+        return "hbm", ((2 if tag[1] else 1) * L * C * esz + 2 * B * N * C * esz + 16 * B * geo["regions"]
+                       + (32 * B * N if tag[4] else 0))
     if name == "vtdge_decompress_layernorm":
         # the scatter-back plus one more write of every token (the next block's first LayerNorm)
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + 3 * B * N * C * esz

@@ -133,11 +133,15 @@ int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *p
  * are found from this block's gate indices `cur_indices` [B, H/R, W/R] (S splits in `splits`, as given to
  * vtdge_index_to_patch) and `offsets` [B+1] instead of the patch list.  Both results are bit-identical to the two
  * separate calls.  next_weight == NULL (with next_bias, next_indices) leaves the router out.  R must be 4 and every
- * split size must divide it; VTDGE_ERR_UNSUPPORTED for another R. */
+ * split size must divide it; VTDGE_ERR_UNSUPPORTED for another R.
+ * out_records (nullable) [B * (extra + H*W), 16] bf16: the statistics record of every row of `out` as stored (mean
+ * and sqrt(var + records_eps), see vtdge_layernorm_stats), for the next block's norm1 -> kv through
+ * vtdge_linear_layernorm; one-pass fp32 sums about a value of the row itself.  bf16 rows of 264 to 512 channels. */
 int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits,
                             const int64_t *offsets, const void *ref, void *out, const void *next_weight,
-                            const void *next_bias, void *next_gate, int64_t *next_indices, int B, int H, int W, int C,
-                            int extra, int R, int S, int S2, int dtype, void *stream);
+                            const void *next_bias, void *next_gate, int64_t *next_indices, void *out_records,
+                            float records_eps, int B, int H, int W, int C, int extra, int R, int S, int S2, int dtype,
+                            void *stream);
 
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */

@@ -770,27 +770,50 @@ __global__ __launch_bounds__(256) void decompress_ln_kernel(const T *__restrict_
 // router sums them, and finishes with the router's Linear + argmax on the NEXT block's gate weights: the indices
 // and logits it leaves are bit for bit those of router_kernel run on `out`, without a second pass over the tokens.
 // The group of a sample's first region also scatters the sample's extra tokens.
-template <typename T, int PS, bool SUB>
+// Statistics record of one stored row from the group's sums of (x - pivot) and (x - pivot)^2, the pivot being a value
+// of the row itself (no cancellation however far the row's mean is from zero).  Values are wave-uniform.
+__device__ __forceinline__ void row_record(float pivot, float s1, float s2, int C, float eps, u32x4 &lo, u32x4 &hi)
+{
+    const float m = s1 / (float)C;
+    const float var = fmaxf(s2 / (float)C - m * m, 0.f);
+    ln_record(pivot + m, sqrtf(var + eps), lo, hi);
+}
+
+// STAT (one wave per region, all 64 lanes present, `act` false for lanes past the row): also writes the
+// statistics records of the 16 stored rows, `rec` pointing at the record of the region's first token.
+template <typename T, int PS, bool SUB, bool STAT = false>
 __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T *__restrict__ sub, int64_t r0,
                                                const T *__restrict__ refp, T *__restrict__ outp, int W, int C,
-                                               float (&acc)[Elem<T>::VEC])
+                                               float (&acc)[Elem<T>::VEC], bool act = true,
+                                               u32x4 *__restrict__ rec = nullptr, float eps = 0.f)
 {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int STEP = 4 / PS;
+    const int lane = threadIdx.x & 63;
 #pragma unroll 1
     for (int dy = 0; dy < 4; dy++) {                       // one token row (4 tokens) at a time; not unrolled: the
                                                            // loads of one row are what a wave keeps in flight
         constexpr int NJ = PS;                              // packed rows these tokens take their values from
         const int j0 = (dy / STEP) * PS;
+        float pivot[4], st[8];
         u32x4 xr[4], ir[NJ], sr[NJ];
+        if constexpr (STAT) {
+            const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int j = 0; j < NJ; j++) {
-            ir[j] = *reinterpret_cast<const u32x4 *>(in + (r0 + j0 + j) * (int64_t)C);
-            if constexpr (SUB) sr[j] = *reinterpret_cast<const u32x4 *>(sub + (r0 + j0 + j) * (int64_t)C);
+            for (int j = 0; j < NJ; j++) ir[j] = sr[j] = z;
+#pragma unroll
+            for (int dx = 0; dx < 4; dx++) xr[dx] = z;
         }
+        if (act) {
 #pragma unroll
-        for (int dx = 0; dx < 4; dx++)
-            xr[dx] = *reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C);
+            for (int j = 0; j < NJ; j++) {
+                ir[j] = *reinterpret_cast<const u32x4 *>(in + (r0 + j0 + j) * (int64_t)C);
+                if constexpr (SUB) sr[j] = *reinterpret_cast<const u32x4 *>(sub + (r0 + j0 + j) * (int64_t)C);
+            }
+#pragma unroll
+            for (int dx = 0; dx < 4; dx++)
+                xr[dx] = *reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C);
+        }
         // in - sub, rounded to the storage type (kept packed: four registers per row)
         if constexpr (SUB) {
 #pragma unroll
@@ -811,22 +834,49 @@ __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T
 #pragma unroll
             for (int c = 0; c < VEC; c++) r[c] += dv[c];
             const u32x4 packed = Elem<T>::pack(r);
-            *reinterpret_cast<u32x4 *>(outp + ((int64_t)dy * W + dx) * C) = packed;
+            if (act) *reinterpret_cast<u32x4 *>(outp + ((int64_t)dy * W + dx) * C) = packed;
             float f[VEC];
             Elem<T>::unpack(packed, f);                   // as stored: what the next block's router reads
 #pragma unroll
             for (int c = 0; c < VEC; c++) acc[c] += f[c];
+            if constexpr (STAT) {
+                pivot[dx] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(f[0])));
+                float a = 0.f, q = 0.f;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    const float d = f[c] - pivot[dx];
+                    a += d;
+                    q += d * d;
+                }
+                st[2 * dx] = act ? a : 0.f;
+                st[2 * dx + 1] = act ? q : 0.f;
+            }
+        }
+        if constexpr (STAT) {
+            wave_sum_n<8>(st);
+            // the four records are 128 contiguous bytes: lane l < 8 writes half l % 2 of token l / 2
+            u32x4 mine = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int dx = 0; dx < 4; dx++) {
+                u32x4 lo, hi;
+                row_record(pivot[dx], st[2 * dx], st[2 * dx + 1], C, eps, lo, hi);
+                if (lane == 2 * dx) mine = lo;
+                if (lane == 2 * dx + 1) mine = hi;
+            }
+            if (lane < 8) rec[(int64_t)dy * W * 2 + lane] = mine;
         }
     }
 }
 
-template <typename T, int GS, bool SUB>
+template <typename T, int GS, bool SUB, bool STAT = false>
 __global__ __launch_bounds__(256) void decompress_route_kernel(
     const T *__restrict__ in, const T *__restrict__ sub, const int64_t *__restrict__ cur_indices,
     const int64_t *__restrict__ splits, const int64_t *__restrict__ offsets, const T *__restrict__ ref,
     T *__restrict__ out, const T *__restrict__ weight, const T *__restrict__ bias, T *__restrict__ gate,
-    int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2)
+    int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2,
+    u32x4 *__restrict__ records = nullptr, float eps = 0.f)
 {
+    static_assert(!STAT || (GS == WAVE && std::is_same<T, bf16_t>::value), "records: one wave per region, bf16 rows");
     constexpr int VEC = Elem<T>::VEC;
     constexpr int R = 4;
     const int lane = threadIdx.x & (GS - 1);
@@ -859,35 +909,61 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
 #pragma unroll
     for (int s = 0; s < VTDGE_MAX_SPLITS; s++) part[s] = 0.f;
     const int64_t tok0 = (int64_t)(ry * R) * W + rx * R + extra;
-    for (int v = lane; v < nvec; v += GS) {
+    // STAT: the host sends rows of at most GS vectors, and every lane makes the one trip (lanes past the row idle
+    // inside it, present for the sums over the wave)
+    const int vend = STAT ? GS : nvec;
+    for (int v0 = lane; v0 < vend; v0 += GS) {
+        const bool act = !STAT || v0 < nvec;
+        const int v = act ? v0 : 0;
         float acc[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) acc[i] = 0.f;
         const int64_t off = ((int64_t)b * N + tok0) * C + v * VEC;
         const T *inv = in + v * VEC;
         const T *subv = SUB ? sub + v * VEC : nullptr;
-        if (ps == 4) region_scatter<T, 4, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
-        else if (ps == 2) region_scatter<T, 2, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
-        else region_scatter<T, 1, SUB>(inv, subv, r0, ref + off, out + off, W, C, acc);
+        u32x4 *rec = STAT ? records + ((int64_t)b * N + tok0) * 2 : nullptr;
+        if (ps == 4) region_scatter<T, 4, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
+        else if (ps == 2) region_scatter<T, 2, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
+        else region_scatter<T, 1, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
         if (rr == 0) {          // the sample's extra tokens: packed rows row_b .. row_b + extra - 1
             for (int e = 0; e < extra; e++) {
                 float d[VEC], r[VEC];
-                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(inv + (row_b + e) * (int64_t)C), d);
-                if constexpr (SUB) {
-                    float sv[VEC];
-                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(subv + (row_b + e) * (int64_t)C), sv);
 #pragma unroll
-                    for (int c = 0; c < VEC; c++) d[c] -= sv[c];
-                    Elem<T>::unpack(Elem<T>::pack(d), d);      // rounded to the storage type
-                }
+                for (int c = 0; c < VEC; c++) d[c] = r[c] = 0.f;
                 const int64_t oe = ((int64_t)b * N + e) * C + v * VEC;
-                Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + oe), r);
+                if (act) {
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(inv + (row_b + e) * (int64_t)C), d);
+                    if constexpr (SUB) {
+                        float sv[VEC];
+                        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(subv + (row_b + e) * (int64_t)C), sv);
+#pragma unroll
+                        for (int c = 0; c < VEC; c++) d[c] -= sv[c];
+                        Elem<T>::unpack(Elem<T>::pack(d), d);      // rounded to the storage type
+                    }
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + oe), r);
+                }
 #pragma unroll
                 for (int c = 0; c < VEC; c++) r[c] += d[c];
-                *reinterpret_cast<u32x4 *>(out + oe) = Elem<T>::pack(r);
+                const u32x4 packed = Elem<T>::pack(r);
+                if (act) *reinterpret_cast<u32x4 *>(out + oe) = packed;
+                if constexpr (STAT) {
+                    float f[VEC], st[2] = {0.f, 0.f};
+                    Elem<T>::unpack(packed, f);
+                    const float pivot = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(f[0])));
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        const float dl = f[c] - pivot;
+                        st[0] += act ? dl : 0.f;
+                        st[1] += act ? dl * dl : 0.f;
+                    }
+                    wave_sum_n<2>(st);
+                    u32x4 lo, hi;
+                    row_record(pivot, st[0], st[1], C, eps, lo, hi);
+                    if (lane < 2) records[((int64_t)b * N + e) * 2 + lane] = lane ? hi : lo;
+                }
             }
         }
-        if (weight != nullptr) {
+        if (weight != nullptr && act) {
 #pragma unroll
             for (int i = 0; i < VEC; i++) acc[i] = Elem<T>::round(acc[i] / (float)(R * R));
 #pragma unroll
@@ -1296,8 +1372,8 @@ extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const
 extern "C" int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices,
                                        const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
                                        const void *next_weight, const void *next_bias, void *next_gate,
-                                       int64_t *next_indices, int B, int H, int W, int C, int extra, int R, int S,
-                                       int S2, int dtype, void *stream)
+                                       int64_t *next_indices, void *out_records, float records_eps, int B, int H,
+                                       int W, int C, int extra, int R, int S, int S2, int dtype, void *stream)
 {
     VT_REQUIRE(in && cur_indices && splits && offsets && ref && out, VTDGE_ERR_ARG, "decompress_router: NULL operand");
     VT_REQUIRE((next_weight == nullptr) == (next_bias == nullptr) && (next_weight == nullptr) == (next_indices == nullptr),
@@ -1315,6 +1391,19 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
     const int gs = group_size(C / (dtype == VTDGE_BF16 ? 8 : 4));
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
+    if (out_records != nullptr) {
+        VT_REQUIRE(dtype == VTDGE_BF16 && gs == WAVE && C / 8 <= WAVE, VTDGE_ERR_UNSUPPORTED,
+                   "decompress_router: statistics records are written for bf16 rows of 264 to 512 channels (C=%d)", C);
+        VT_REQUIRE(aligned16(out_records), VTDGE_ERR_ARG, "decompress_router: records must be 16-byte aligned");
+#define VT_STAT(SUBF)                                                                                                \
+    decompress_route_kernel<bf16_t, WAVE, SUBF, true><<<grid, block, 0, st>>>(                                       \
+        (const bf16_t *)in, (const bf16_t *)sub, cur_indices, splits, offsets, (const bf16_t *)ref, (bf16_t *)out,   \
+        (const bf16_t *)next_weight, (const bf16_t *)next_bias, (bf16_t *)next_gate, next_indices, B, H, W, C, extra, \
+        S, S2, (u32x4 *)out_records, records_eps)
+        if (sub) VT_STAT(true); else VT_STAT(false);
+#undef VT_STAT
+        return check_launch("decompress_router");
+    }
 #define VT_LAUNCH2(T, GS, SUBF)                                                                                    \
     decompress_route_kernel<T, GS, SUBF><<<grid, block, 0, st>>>(                                                  \
         (const T *)in, (const T *)sub, cur_indices, splits, offsets, (const T *)ref, (T *)out,                     \

@@ -188,9 +188,16 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         out, handed["x_ln"] = ops.decompress_layernorm(q2, patches, x, W, extra, nn1.weight, nn1.bias, nn1.eps,
                                                        sub=comp, rows_dev=rows_dev, rows=cap)
     elif nxt is not None and FUSE_NEXT_ROUTER and R == 4 and nxt.region_size == 4:
-        out, ngate, nidx = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
-                                                 next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias)
+        nattn = next_block.attn
+        want_stats = (FOLD_NORMS and getattr(nattn, "sr_ratio", 1) <= 1 and ops.fits_scatter_stats(x)
+                      and ops.fits_linear_layernorm(x, nattn.kv.weight))
+        res = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
+                                    next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias,
+                                    stats_eps=next_block.norm1.eps if want_stats else None)
+        out, ngate, nidx = res[:3]
         handed["routed"] = (ngate, nidx)
+        if want_stats:
+            handed["x_stats"] = res[3]
     else:
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 

@@ -175,9 +175,10 @@ def decompress_layernorm(inp, patches, reference, width, num_extra_tokens, ln_we
 
 
 def decompress_router(inp, indices, splits, offsets, reference, H, W, region_size, sub=None, next_weight=None,
-                      next_bias=None, want_gate=True):
+                      next_bias=None, want_gate=True, stats_eps=None):
     """Scatter (inp - sub) + reference back over the tokens by region, and route the NEXT block on the result:
-    -> (out, next_gate or None, next_indices or None).  `indices` [B, Hr, Wr] are this block's gate indices, `offsets`
+    -> (out, next_gate or None, next_indices or None), and with `stats_eps` (a LayerNorm's eps; bf16 rows of 264 to
+    512 channels) a fourth value: the statistics records of the rows of `out` for `linear_layernorm`.  `indices` [B, Hr, Wr] are this block's gate indices, `offsets`
     [B+1] the prefix of its query counts.  The three outputs equal decompress(...) and router(out, next_weight,
     next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75."""
     _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
@@ -206,10 +207,22 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
         Hr, Wr = H // region_size, W // region_size
         gate = torch.empty((B, Hr, Wr, S2), dtype=inp.dtype, device=inp.device) if want_gate else None
         nidx = torch.empty((B, Hr, Wr), dtype=torch.int64, device=inp.device)
+    rec = None
+    if stats_eps is not None:
+        rec = torch.empty((B * N, 16), dtype=torch.bfloat16, device=inp.device)
     call("vtdge_decompress_router", ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference),
-         ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), B, H, W, C, extra, region_size, S, S2,
-         dtype_code(inp), stream_ptr(), tag=("decompress_router", sub is not None, next_weight is not None, C))
+         ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), ptr(rec),
+         float(stats_eps if stats_eps is not None else 0.0), B, H, W, C, extra, region_size, S, S2,
+         dtype_code(inp), stream_ptr(),
+         tag=("decompress_router", sub is not None, next_weight is not None, C, rec is not None))
+    if stats_eps is not None:
+        return out, gate, nidx, rec
     return out, gate, nidx
+
+
+def fits_scatter_stats(x):
+    """Whether `decompress_router` can write statistics records for rows like those of x [B, N, C]."""
+    return x.is_cuda and x.dtype == torch.bfloat16 and 264 <= x.shape[-1] <= 512 and x.shape[-1] % 8 == 0
 
 
 def fits_decompress_layernorm(x):
