@@ -194,6 +194,14 @@ int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void
  *                           may be anything), else VTDGE_ERR_UNSUPPORTED.
  * Against vtdge_layernorm followed by vtdge_linear the result differs by the rounding of W' instead of that of
  * LayerNorm(a) to bf16: the same order of magnitude, not the same bits. */
+/* vtdge_linear (no activation) that also writes the statistics records of its output rows, for a
+ * vtdge_linear_layernorm that takes `out` next: proj + residual followed by norm2 -> fc1
+ * (vtpack/models/dge/deit_dge.py:96, :128, :38-44).  The records are computed from the fp32 sums before their rounding
+ * to bf16.  Weight-stationary kernel with one column group only: bf16, K = 384, N = 384, rows >= 2048. */
+int vtdge_linear_stats(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,
+                       const void *residual, int64_t ldr, void *out, int64_t ldo, void *out_records,
+                       float records_eps, const int64_t *rows_dev, int64_t rows, int N, int K, int dtype,
+                       void *stream);
 int vtdge_layernorm_stats(const void *x, void *records, const int64_t *rows_dev, int64_t rows, int C, float eps,
                           int dtype, void *stream);
 int vtdge_layernorm_fold(const void *W, const void *bias, const void *ln_weight, const void *ln_bias, int N, int K,

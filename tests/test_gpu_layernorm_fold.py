@@ -1,0 +1,344 @@
+"""LayerNorm folded into the Linear behind it (norm1 -> kv, norm2 -> fc1; vtpack/models/dge/deit_dge.py:127-128 with
+:73 and :38-44): the statistics records and their three producers, the Linear that consumes them, and the model with
+the folding on and off.
+
+The reference for every value is torch in fp64 on the same bf16 inputs: F.layer_norm followed by a matrix product
+(+ GELU).  Inputs are scaled so that expected values stay below 4 in magnitude, where the plain 2e-2 max-abs bar of
+the bf16 tests applies.
+"""
+import pytest
+import torch
+
+from util import BF16_ABS, SPLITS, abs_err, random_indices
+
+pytestmark = pytest.mark.gpu
+
+C = 384
+EPS = 1e-6
+
+
+def decode(rec):
+    """records [rows, 16] bf16 -> (mean, sigma) as the consuming kernel sums them, and the raw values."""
+    r = rec.float()
+    return r[:, 0] + r[:, 2] + r[:, 5], r[:, 6] + r[:, 7], r
+
+
+def assert_record_layout(rec):
+    """lo = (m1, m1, m2, m1, m2, m3, s1, s2), hi = (s1, s2, 0, ...): what one MFMA K step multiplies by the column
+    record (-c1, -c2, -c1, -c3, -c2, -c1, b1, b1 | b2, 0, ...)."""
+    r = rec.float()
+    assert bool((r[:, 0] == r[:, 1]).all() and (r[:, 0] == r[:, 3]).all() and (r[:, 2] == r[:, 4]).all())
+    assert bool((r[:, 6] == r[:, 8]).all() and (r[:, 7] == r[:, 9]).all() and (r[:, 10:] == 0).all())
+
+
+def want_stats(x):
+    xd = x.double().reshape(-1, x.shape[-1])
+    return xd.mean(1), (xd.var(1, unbiased=False) + EPS).sqrt()
+
+
+def rows_like_tokens(M, seed, shift=0.0, dev="cuda"):
+    """Rows with per-row scale between 0.5 and 2.5 and a per-row offset of `shift` standard deviations."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, C, generator=g) * (0.5 + 2 * torch.rand(M, 1, generator=g))
+    return (x + shift * torch.randn(M, 1, generator=g)).bfloat16().to(dev)
+
+
+def layer(N, seed, dev):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(N, C, generator=g) * 0.03).bfloat16().to(dev)
+    b = (torch.randn(N, generator=g) * 0.2).bfloat16().to(dev)
+    gamma = (1 + 0.3 * torch.randn(C, generator=g)).bfloat16().to(dev)
+    beta = (0.2 * torch.randn(C, generator=g)).bfloat16().to(dev)
+    return w, b, gamma, beta
+
+
+def want_linear_layernorm(x, w, b, gamma, beta, act):
+    y = torch.nn.functional.layer_norm(x.double(), (C,), gamma.double(), beta.double(), EPS)
+    want = y @ w.double().T + (b.double() if b is not None else 0.0)
+    return torch.nn.functional.gelu(want) if act == "gelu" else want
+
+
+# ----------------------------------------------------------------------------- records from the statistics kernel
+@pytest.mark.parametrize("shift", [0.0, 3.0, 200.0])
+@pytest.mark.parametrize("live", [None, 0, 1, 5, 4097])
+def test_statistics_records(dev, live, shift):
+    from vtpack_amd import ops
+    M = 5000
+    x = rows_like_tokens(M, 11, shift, dev)
+    rows_dev = None if live is None else torch.tensor([live], dtype=torch.int64, device=dev)
+    rec = torch.full((M, 16), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.layernorm_stats(x, EPS, rows_dev=rows_dev, out=rec)
+    L = M if live is None else live
+    assert bool((rec[L:] == 7.0).all())
+    if L:
+        mean, sigma, _ = decode(rec[:L])
+        m_ref, s_ref = want_stats(x[:L])
+        assert_record_layout(rec[:L])
+        # mean to fp32 accuracy relative to the row's magnitude (three bf16 parts), sigma to 2^-16 (two parts)
+        assert float(((mean.double().cpu() - m_ref.cpu()).abs() / x[:L].double().abs().amax(1).cpu()).max()) < 1e-6
+        assert float(((sigma.double().cpu() - s_ref.cpu()) / s_ref.cpu()).abs().max()) < 2e-5
+
+
+# ----------------------------------------------------------------------------- the consuming Linear
+@pytest.mark.parametrize("live", [None, 0, 1, 7, 31, 32, 33, 63, 65, 2047, 2500])
+@pytest.mark.parametrize("N,act", [(768, "none"), (1536, "gelu"), (384, "none")])
+@pytest.mark.parametrize("packed", [True, False])
+def test_linear_layernorm_live_rows(dev, live, N, act, packed):
+    from vtpack_amd import ops
+    M = 2600
+    x = rows_like_tokens(M, 3 + (live or 0), 1.0, dev)
+    w, b, gamma, beta = layer(N, 5, dev)
+    rows_dev = None if live is None else torch.tensor([live], dtype=torch.int64, device=dev)
+    L = M if live is None else live
+    rec = ops.layernorm_stats(x, EPS, rows_dev=rows_dev)
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.PACK_WEIGHTS = packed
+    try:
+        ops.invalidate_packed()
+        ops.linear_layernorm(x, rec, w, b, gamma, beta, act=act, rows_dev=rows_dev, out=out)
+    finally:
+        ops.PACK_WEIGHTS = True
+        ops.invalidate_packed()
+    if L:
+        want = want_linear_layernorm(x[:L], w, b, gamma, beta, act)
+        assert float(want.abs().max()) < 4.0
+        assert abs_err(out[:L], want) <= BF16_ABS
+    assert bool((out[L:] == 7.0).all())
+
+
+@pytest.mark.parametrize("shift", [0.0, 30.0, 100.0])
+def test_linear_layernorm_rows_far_from_zero(dev, shift):
+    """Rows whose mean is up to a few hundred standard deviations from zero: the rank-one correction
+    mean * colsum(W') is as large as the product itself and cancels it to fp32 accuracy, so the error stays that of
+    the two-kernel path.  (What is left of the cancellation is the fp32 rounding of the product, about
+    2^-22 |mean| sum|W'|, times rstd: it reaches the bf16 bar only where |mean| / sigma passes ~10^4, i.e. for rows
+    that bf16 cannot tell from constant ones.)"""
+    from vtpack_amd import ops
+    M, N = 4096, 768
+    x = rows_like_tokens(M, 21, shift, dev)
+    _, s_ref = want_stats(x)
+    keep = (x.double().mean(1).abs() / s_ref) < 1e3          # drop rows that rounding has made constant
+    x = x[keep][:2304 + (int(keep.sum()) - 2304) // 32 * 32].contiguous()
+    w, b, gamma, beta = layer(N, 22, dev)
+    got = ops.linear_layernorm(x, ops.layernorm_stats(x, EPS), w, b, gamma, beta)
+    two = ops.linear(ops.layernorm(x, gamma, beta, EPS), w, b)
+    want = want_linear_layernorm(x, w, b, gamma, beta, "none")
+    assert float(want.abs().max()) < 4.0
+    assert abs_err(got, want) <= BF16_ABS
+    assert abs_err(got, want) <= 1.25 * abs_err(two, want) + 2 ** -9
+
+
+def test_linear_layernorm_of_zero_rows_is_the_folded_bias(dev):
+    """All-zero rows (padding): LayerNorm gives beta, the Linear bias + W beta, and the folded form reproduces it
+    through sigma * b' * rstd with no product to cancel."""
+    from vtpack_amd import ops
+    M, N = 2304, 768
+    x = rows_like_tokens(M, 5, 0.0, dev)
+    x[::7] = 0
+    w, b, gamma, beta = layer(N, 6, dev)
+    got = ops.linear_layernorm(x, ops.layernorm_stats(x, EPS), w, b, gamma, beta)
+    want = want_linear_layernorm(x, w, b, gamma, beta, "none")
+    assert abs_err(got[::7], want[::7]) <= 2 ** -8 * float(want[::7].abs().max())     # one bf16 rounding
+    assert abs_err(got, want) <= BF16_ABS
+
+
+def test_linear_layernorm_full_shapes_and_repeatable(dev):
+    """The two shapes of the headline model (kv: 65 792 x 768, fc1 + GELU: ~27 000 live rows x 1536) and bit-equal
+    repeats."""
+    from vtpack_amd import ops
+    for M, N, act, live in ((65792, 768, "none", None), (65792, 1536, "gelu", 27113)):
+        x = rows_like_tokens(M, M % 97, 0.5, dev)
+        w, b, gamma, beta = layer(N, N, dev)
+        rows_dev = None if live is None else torch.tensor([live], dtype=torch.int64, device=dev)
+        L = M if live is None else live
+        rec = ops.layernorm_stats(x, EPS, rows_dev=rows_dev)
+        first = ops.linear_layernorm(x, rec, w, b, gamma, beta, act=act, rows_dev=rows_dev)
+        want = want_linear_layernorm(x[:L], w, b, gamma, beta, act)
+        assert float(want.abs().max()) < 4.0
+        assert abs_err(first[:L], want) <= BF16_ABS
+        for _ in range(2):
+            assert torch.equal(ops.linear_layernorm(x, rec, w, b, gamma, beta, act=act, rows_dev=rows_dev)[:L], first[:L])
+
+
+def test_folded_weights_follow_edits(dev):
+    """The folded copy is keyed on all four tensors: an in-place edit of the LayerNorm's scale or of the Linear's bias
+    is seen at the next call; a write through .data needs invalidate_packed."""
+    from vtpack_amd import ops
+    M, N = 2304, 768
+    x = rows_like_tokens(M, 1, 0.0, dev)
+    w, b, gamma, beta = layer(N, 2, dev)
+    rec = ops.layernorm_stats(x, EPS)
+
+    def check():
+        got = ops.linear_layernorm(x, rec, w, b, gamma, beta)
+        assert abs_err(got, want_linear_layernorm(x, w, b, gamma, beta, "none")) <= BF16_ABS
+        return got
+
+    base = check()
+    gamma.mul_(0.5)
+    assert not torch.equal(check(), base)
+    b.add_(0.25)
+    check()
+    w.data.mul_(0.5)                       # not counted by torch
+    ops.invalidate_packed(w)
+    check()
+
+
+def test_operand_checks(dev):
+    from vtpack_amd import ops
+    x = rows_like_tokens(2304, 1, 0.0, dev)
+    w, b, gamma, beta = layer(768, 2, dev)
+    rec = ops.layernorm_stats(x, EPS)
+    with pytest.raises(TypeError):
+        ops.layernorm_stats(x.float(), EPS)
+    with pytest.raises(ValueError):
+        ops.linear_layernorm(x, rec[:100], w, b, gamma, beta)
+    with pytest.raises(ValueError):
+        ops.linear_layernorm(x[:100], rec[:100], w, b, gamma, beta)            # too few rows for the kernel
+    with pytest.raises(TypeError):
+        ops.linear_layernorm(x, rec, w, b, gamma.float(), beta)
+    with pytest.raises(ValueError):
+        ops.linear_layernorm(x, rec, w, b, gamma[:100], beta[:100])
+    with pytest.raises(ValueError):
+        ops.linear(x, w, b, stats_eps=EPS)                                     # records need N = 384
+    assert not ops.fits_linear_layernorm(x.float(), w)
+    assert not ops.fits_linear_layernorm(x, torch.zeros(100, C, dtype=torch.bfloat16, device=dev))
+
+
+# ----------------------------------------------------------------------------- records from the producing kernels
+@pytest.mark.parametrize("live", [None, 0, 17, 33, 64, 2599])
+@pytest.mark.parametrize("has_bias,has_res", [(True, True), (True, False), (False, True), (False, False)])
+def test_linear_writes_records_of_its_rows(dev, live, has_bias, has_res):
+    """proj + residual with the records of its output rows: the output is the plain Linear's bit for bit, the records
+    are the statistics of the fp32 sums."""
+    from vtpack_amd import ops
+    M = 2600
+    g = torch.Generator().manual_seed(7 + (live or 0))
+    a = torch.randn(M, C, generator=g).bfloat16().to(dev)
+    w = (torch.randn(C, C, generator=g) * 0.05).bfloat16().to(dev)
+    b = (torch.randn(C, generator=g) * 0.2).bfloat16().to(dev) if has_bias else None
+    res = (torch.randn(M, C, generator=g) * 2 + 3 * torch.randn(M, 1, generator=g)).bfloat16().to(dev) if has_res else None
+    rows_dev = None if live is None else torch.tensor([live], dtype=torch.int64, device=dev)
+    L = M if live is None else live
+    plain = ops.linear(a, w, b, residual=res, rows_dev=rows_dev)
+    out, rec = ops.linear(a, w, b, residual=res, rows_dev=rows_dev, stats_eps=EPS)
+    assert torch.equal(out[:L], plain[:L])
+    if not L:
+        return
+    want = a[:L].double() @ w.double().T
+    if has_bias:
+        want = want + b.double()
+    if has_res:
+        want = want + res[:L].double()
+    mean, sigma, _ = decode(rec[:L])
+    m_ref, s_ref = want_stats(want)
+    assert_record_layout(rec[:L])
+    assert float((mean.double() - m_ref).abs().max()) < 1e-5
+    assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
+
+
+def test_linear_records_at_full_size_feed_the_next_linear(dev):
+    """proj -> (records) -> fc1 at the headline shape, against LayerNorm of the stored rows in fp64."""
+    from vtpack_amd import ops
+    M, live = 65792, 27113
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(M, C, generator=g).bfloat16().to(dev)
+    wp = (torch.randn(C, C, generator=g) * 0.05).bfloat16().to(dev)
+    res = torch.randn(M, C, generator=g).bfloat16().to(dev)
+    w1, b1, gamma, beta = layer(1536, 9, dev)
+    rows_dev = torch.tensor([live], dtype=torch.int64, device=dev)
+    q1, rec = ops.linear(a, wp, None, residual=res, rows_dev=rows_dev, stats_eps=EPS)
+    hid = ops.linear_layernorm(q1, rec, w1, b1, gamma, beta, act="gelu", rows_dev=rows_dev)
+    want = want_linear_layernorm(q1[:live], w1, b1, gamma, beta, "gelu")
+    assert float(want.abs().max()) < 4.0
+    assert abs_err(hid[:live], want) <= BF16_ABS
+
+
+@pytest.mark.parametrize("B,H,Cc,extra", [(8, 16, 384, 1), (4, 32, 384, 2), (3, 8, 512, 0), (2, 8, 264, 1)])
+def test_scatter_back_writes_records_of_the_tokens(dev, B, H, Cc, extra):
+    from vtpack_amd import ops
+    W = H
+    N = extra + H * W
+    g = torch.Generator().manual_seed(B)
+    idx = torch.from_numpy(random_indices(B, B, H // 4, W // 4)).to(dev)
+    splits = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    patches, offsets, lengths = ops.index_to_patch(idx, splits, 4, extra, capacity=B * N)
+    x = (torch.randn(B, N, Cc, generator=g) * 2 + 5 * torch.randn(B, N, 1, generator=g)).bfloat16().to(dev)
+    q = torch.randn(B * N, Cc, generator=g).bfloat16().to(dev)
+    sub = torch.randn(B * N, Cc, generator=g).bfloat16().to(dev)
+    wgt = (torch.randn(3, Cc, generator=g) * 0.1).bfloat16().to(dev)
+    bias = torch.zeros(3, dtype=torch.bfloat16, device=dev)
+    o0, g0, i0 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt, next_bias=bias)
+    o1, g1, i1, rec = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt,
+                                            next_bias=bias, stats_eps=EPS)
+    assert torch.equal(o0, o1) and torch.equal(g0, g1) and torch.equal(i0, i1)
+    mean, sigma, _ = decode(rec)
+    m_ref, s_ref = want_stats(o1)
+    assert_record_layout(rec)
+    assert float((mean.double() - m_ref).abs().max()) < 5e-6 * float(o1.double().abs().max())
+    assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
+    # without the next router as well
+    o2, _, _, rec2 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=None, stats_eps=EPS)
+    m2, s2, _ = decode(rec2)
+    m_ref2, s_ref2 = want_stats(o2)
+    assert float(((s2.double() - s_ref2) / s_ref2).abs().max()) < 3e-5
+
+
+def test_scatter_records_refused_for_other_rows(dev):
+    from vtpack_amd import ops
+    from vtpack_amd._lib import VtdgeError
+    B, H, Cc = 2, 8, 192
+    idx = torch.zeros(B, 2, 2, dtype=torch.int64, device=dev)
+    splits = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    patches, offsets, lengths = ops.index_to_patch(idx, splits, 4, 1, capacity=B * 65)
+    x = torch.zeros(B, 65, Cc, dtype=torch.bfloat16, device=dev)
+    q = torch.zeros(B * 65, Cc, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(VtdgeError):
+        ops.decompress_router(q, idx, splits, offsets, x, H, H, 4, stats_eps=EPS)
+    assert not ops.fits_scatter_stats(x) and not ops.fits_scatter_stats(x.float())
+
+
+# ----------------------------------------------------------------------------- the model with and without
+def test_model_with_and_without_folded_norms(dev):
+    """DeiT-S+DGE, bf16, 256 px, batch 16 (enough rows for the weight-stationary kernels): with the folding on the
+    forward launches one statistics kernel (the first block's tokens) and one LayerNorm (the final one) instead of 25
+    LayerNorms; the routing of the first block is the same either way and, while the routing stays the same, the
+    logits agree within the bf16 bar."""
+    from vtpack_amd import _lib, engine
+    from vtpack_amd.models import dge as zoo
+    from vtpack_amd.synthetic import set_synthetic_router, synthetic_images
+
+    class Count:
+        def __init__(self):
+            self.names = []
+
+        def begin(self, name, tag):
+            self.names.append(name)
+
+        def end(self):
+            pass
+
+    torch.manual_seed(0)
+    m = zoo.deit_dge_s124_small_patch16_256()
+    set_synthetic_router(m, 0)
+    m = m.eval().to(dev).to(torch.bfloat16)
+    img = synthetic_images(16, 256, seed=0, dtype=torch.bfloat16, device=dev)
+    runs = {}
+    try:
+        for fold in (True, False):
+            engine.FOLD_NORMS = fold
+            _lib.timer = Count()
+            with torch.no_grad():
+                out = m(img)
+            runs[fold] = (out.float(), [blk.dge.states["batches_device"].clone() for blk in m.blocks], _lib.timer.names)
+    finally:
+        engine.FOLD_NORMS = True
+        _lib.timer = None
+    (on, len_on, names_on), (off, len_off, names_off) = runs[True], runs[False]
+    assert names_off.count("vtdge_layernorm") == 25 and names_off.count("vtdge_linear_layernorm") == 0
+    assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 1
+    assert names_on.count("vtdge_linear_layernorm") == 24 and names_on.count("vtdge_linear_stats") == 12
+    assert bool(torch.isfinite(on).all())
+    assert torch.equal(len_on[0], len_off[0])
+    if all(torch.equal(a, b) for a, b in zip(len_on, len_off)):
+        assert abs_err(on, off) <= 2 * BF16_ABS

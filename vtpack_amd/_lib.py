@@ -39,6 +39,7 @@ SIGNATURES = {
     "vtdge_linear_packed_size": [_i, _i, _i, _p],
     "vtdge_linear_prepack": [_p, _i, _i, _i, _p, _p],
     "vtdge_linear_prepacked": [_p, _l, _p, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],
+    "vtdge_linear_stats": [_p, _l, _p, _p, _p, _p, _l, _p, _l, _p, _f, _p, _l, _i, _i, _i, _p],
     "vtdge_layernorm_stats": [_p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_layernorm_fold": [_p, _p, _p, _p, _i, _i, _i, _p, _p, _p],
     "vtdge_linear_layernorm": [_p, _l, _p, _p, _p, _p, _p, _l, _p, _l, _i, _i, _i, _i, _p],

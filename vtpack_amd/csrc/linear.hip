@@ -195,6 +195,9 @@ int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, 
 int launch_linear_ws_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
                         const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
                         hipStream_t st);
+int launch_linear_ws_stats(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                           int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows,
+                           void *records, float eps, hipStream_t st);
 
 // K-split weight-stationary variant for bf16, K = 1536, narrow N (linear_ks.hip)
 bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
@@ -327,6 +330,26 @@ extern "C" int vtdge_linear_layernorm(const void *A, int64_t lda, const void *ro
                "(rows=%lld N=%d K=%d dtype=%d)", (long long)rows, N, K, dtype);
     return launch_linear_ws_ln(A, lda, row_records, W_folded, packed, col_records, out, ldo, rows_dev, rows, N, act,
                                (hipStream_t)stream);
+}
+
+extern "C" int vtdge_linear_stats(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,
+                                  const void *residual, int64_t ldr, void *out, int64_t ldo, void *out_records,
+                                  float records_eps, const int64_t *rows_dev, int64_t rows, int N, int K, int dtype,
+                                  void *stream)
+{
+    VT_REQUIRE(A && W && out && out_records, VTDGE_ERR_ARG, "linear_stats: NULL operand");
+    VT_REQUIRE(rows >= 0 && N > 0 && K > 0, VTDGE_ERR_ARG, "linear_stats: bad sizes rows=%lld N=%d K=%d",
+               (long long)rows, N, K);
+    VT_REQUIRE(lda >= K && ldo >= N && (!residual || ldr >= N), VTDGE_ERR_ARG, "linear_stats: leading dim too small");
+    VT_REQUIRE((((uintptr_t)A | (uintptr_t)W | (uintptr_t)packed | (uintptr_t)out_records) & 15) == 0, VTDGE_ERR_ARG,
+               "linear_stats: operands must be 16-byte aligned");
+    VT_REQUIRE(dtype == VTDGE_BF16 && N == 384 &&
+                   linear_ws_applicable(lda, ldr, ldo, rows, N, K, 2, VTDGE_ACT_NONE, bias, residual, out),
+               VTDGE_ERR_UNSUPPORTED,
+               "linear_stats: built for bf16, K = 384, N = 384 and 2048 rows or more (rows=%lld N=%d K=%d dtype=%d)",
+               (long long)rows, N, K, dtype);
+    return launch_linear_ws_stats(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, out_records,
+                                  records_eps, (hipStream_t)stream);
 }
 
 extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,

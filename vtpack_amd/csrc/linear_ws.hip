@@ -102,12 +102,19 @@ __device__ __forceinline__ void gelu_part3(EpiUnit &u)
 // fragment the column's record of -colsum(W') and b' in the matching order (`lnw`, two 16-byte halves per output
 // column).  The records of a tile arrive in LDS with the tile (one more direct load, issued by wave 0); the
 // epilogue multiplies by rstd = 1 / (sigma_1 + sigma_2).  A separate bias is not taken (it is part of b').
-template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES, bool HAS_LN = false>
+//
+// HAS_STAT (one column group, i.e. N = 384: the workgroup owns whole output rows): also writes the statistics record
+// of every output row (fp32 values before their rounding to bf16), for a HAS_LN Linear that takes `out` next.  A
+// lane sums its 48 elements of the row about the first of them while the epilogue units pass; the eight partial sums
+// of a row (two lane halves, four waves) meet in LDS and, one step later, sixteen lanes per wave merge them for eight
+// rows each (pairwise-exact merge of means and squared deviations) and write 256 contiguous bytes of records.
+template <int KS, int NB, int ACT, bool HAS_BIAS, bool HAS_RES, bool HAS_LN = false, bool HAS_STAT = false>
 __global__ __launch_bounds__(256) void linear_ws_kernel(
     const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
     const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
     const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp,
-    const u32x4 *__restrict__ lnrec = nullptr, const u32x4 *__restrict__ lnw = nullptr)
+    const u32x4 *__restrict__ lnrec = nullptr, const u32x4 *__restrict__ lnw = nullptr,
+    u32x4 *__restrict__ stat_out = nullptr, float stat_eps = 0.f)
 {
     constexpr int KB = KS * 32;                 // bytes of one operand row
     constexpr int TILE = 32 * KB;               // bytes of one 32-row tile (A, W block or residual) in LDS
@@ -134,6 +141,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     static_assert(EARLY <= PA && 2 * NL <= KS, "prologue / direct loads inside the K loop");
     constexpr int OFF_R = DA * TILE;
     constexpr int OFF_L = 6 * TILE;             // statistics records of the tiles in the A ring, 1 KB each
+    constexpr int OFF_S = OFF_L + (HAS_LN ? DA * 1024 : 0);   // HAS_STAT: two buffers of 8 x 32 partial sums, 16 B each
     static_assert(!(HAS_LN && HAS_BIAS), "with HAS_LN the bias is part of the column records");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -354,6 +362,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     // (8q + e, 8q + 4 + e) of block j into elements e and 4 + e of the lane's 8-column vector (j, q).
     uint32_t e_w[4];        // packed pairs of the current vector
     float rs_prev = 1.0f;   // HAS_LN: rstd of the lane's row in the tile whose epilogue is due
+    float st_p = 0.f, st_a = 0.f, st_q = 0.f;   // HAS_STAT: pivot, sum and sum of squares about it (48 elements)
     float h0, h1;           // elements of an even unit waiting for their odd neighbours
     EpiUnit un;
     auto epi_part1 = [&](auto pp_tag, int n) {
@@ -371,6 +380,48 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
     };
     auto epi_part2 = [&](int n) {
         if constexpr (ACT == VTDGE_ACT_GELU) gelu_part2(un);
+        if constexpr (HAS_STAT && ACT == VTDGE_ACT_NONE) {
+            if (n == 0) {
+                st_p = un.f0;
+                st_a = st_q = 0.f;
+            }
+            const float d0 = un.f0 - st_p, d1 = un.f1 - st_p;
+            st_a += d0;
+            st_q = fmaf(d0, d0, st_q);
+            st_a += d1;
+            st_q = fmaf(d1, d1, st_q);
+        }
+    };
+    // the lane's partial sums of tile t go to LDS ...
+    auto stat_put = [&](int t) {
+        const u32x4 v = {__float_as_uint(st_p), __float_as_uint(st_a), __float_as_uint(st_q), 0u};
+        *reinterpret_cast<u32x4 *>(smem + OFF_S + (t & 1) * 4096 + ((w * 2 + lg) * 32 + lr) * 16) = v;
+    };
+    // ... and, once every wave's are there (a barrier later), become the records of the tile's rows: wave w merges rows
+    // 8w .. 8w+7, lane l < 16 writing half l % 2 of row 8w + l / 2
+    auto stat_finish = [&](int t) {
+        const int row = w * 8 + ((lane >> 1) & 7);
+        const unsigned char *pb = smem + OFF_S + (t & 1) * 4096 + row * 16;
+        float mi[8], m2 = 0.f, ms = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const u32x4 pv = *reinterpret_cast<const u32x4 *>(pb + i * 512);
+            const float a = __uint_as_float(pv.y) * (1.0f / 48.0f);
+            mi[i] = __uint_as_float(pv.x) + a;
+            m2 += __uint_as_float(pv.z) - __uint_as_float(pv.y) * a;
+            ms += mi[i];
+        }
+        const float mean = ms * 0.125f;
+        float dev = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) dev = fmaf(mi[i] - mean, mi[i] - mean, dev);
+        const float var = fmaxf((m2 + 48.0f * dev) * (1.0f / 384.0f), 0.f);
+        u32x4 lo, hi;
+        ln_record(mean, sqrtf(var + stat_eps), lo, hi);
+        int gm = tile_row0(t) + row;
+        gm = gm < M32 ? gm : M32 - 1;
+        if (lane < 16) stat_out[(int64_t)gm * 2 + (lane & 1)] = (lane & 1) ? hi : lo;
+        issued += 1;
     };
     auto epi_part3 = [&](int n, unsigned char *orow) {
         const int j = n / 8, q = (n / 4) % 2, e = n % 4;
@@ -417,7 +468,11 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         using PQ = std::integral_constant<int, 1 - PP>;
         const bool more = k + 1 < nt;
         wait_step(k);
+        if constexpr (HAS_STAT) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the partial sums put last step
         block_barrier();   // what was awaited is in LDS for every wave; the slots read last step are free
+        if constexpr (HAS_STAT) {
+            if (k >= 2) stat_finish(k - 2);
+        }
 
         // Direct loads of this step: the residual of tile k+PR and A(k+PA), six each per wave.  The waves take turns
         // (wave w issues in substeps 6w .. 6w+5: load number s of each tile in substep s, the residual's first), so
@@ -509,6 +564,7 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if constexpr (HAS_STAT && EPI) stat_put(k - 1);
         if constexpr (HAS_LN) {
 #pragma unroll
             for (int j = 0; j < NB; j++) mma_v_fresh(acc[PP][j], wl[j], fl);
@@ -568,6 +624,12 @@ __global__ __launch_bounds__(256) void linear_ws_kernel(
         epi_part2(n);
         epi_part3(n, orow);
     }
+    if constexpr (HAS_STAT) {
+        stat_put(nt - 1);
+        lds_barrier();          // the sums of the last two tiles are in LDS for every wave
+        if (nt >= 2) stat_finish(nt - 2);
+        stat_finish(nt - 1);
+    }
 }
 
 // ----------------------------------------------------------------------------- host
@@ -582,15 +644,16 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
            (((uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15) == 0;
 }
 
-template <int ACT, bool HB, bool HR, bool LN = false>
+template <int ACT, bool HB, bool HR, bool LN = false, bool STAT = false>
 static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
                  int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, hipStream_t st,
-                 const void *lnrec = nullptr, const void *lnw = nullptr)
+                 const void *lnrec = nullptr, const void *lnw = nullptr, void *stat_out = nullptr, float stat_eps = 0.f)
 {
     constexpr int KS = 24, NB = 3;
-    constexpr size_t lds = (size_t)6 * 32 * KS * 32 + (LN ? 4 * 1024 : 0);   // six 32-row tiles (+ four tiles' records)
+    // six 32-row tiles (+ four tiles' records) (+ two buffers of partial sums)
+    constexpr size_t lds = (size_t)6 * 32 * KS * 32 + (LN ? 4 * 1024 : 0) + (STAT ? 2 * 4096 : 0);
     static_assert(lds <= 160 * 1024, "LDS budget");
-    auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR, LN>;
+    auto kern = linear_ws_kernel<KS, NB, ACT, HB, HR, LN, STAT>;
     VT_RESERVE_LDS(kern, lds, "linear");
     const int groups = N / (4 * NB * 32);
     // one workgroup per CU; the P workgroups of a column group are spread over the 8 XCDs, and the workgroups
@@ -601,8 +664,24 @@ static int go_ws(const void *A, int64_t lda, const void *W, const void *Wp, cons
     dim3 grid((unsigned)(P * groups)), block(256);
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
                                    ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp,
-                                   (const u32x4 *)lnrec, (const u32x4 *)lnw);
+                                   (const u32x4 *)lnrec, (const u32x4 *)lnw, (u32x4 *)stat_out, stat_eps);
     return check_launch("linear");
+}
+
+// out = A W^T + bias + residual for N = 384, with the statistics records of the rows of out
+int launch_linear_ws_stats(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                           int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows,
+                           void *records, float eps, hipStream_t st)
+{
+    const bool hb = bias != nullptr, hr = res != nullptr;
+#define VT_WS(HB, HR)                                                                                               \
+    return go_ws<VTDGE_ACT_NONE, HB, HR, false, true>(A, lda, W, Wp, bias, res, ldr, out, ldo, rows_dev, rows, 384, st, \
+                                                      nullptr, nullptr, records, eps)
+    if (hb && hr) VT_WS(true, true);
+    if (hb) VT_WS(true, false);
+    if (hr) VT_WS(false, true);
+    VT_WS(false, false);
+#undef VT_WS
 }
 
 // out = act(LayerNorm(A) W^T + bias) from the raw rows, their statistics records and the folded weights

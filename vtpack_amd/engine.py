@@ -170,10 +170,14 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
             if t is not None:
                 t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
-    q1 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev)
+    fold2 = FOLD_NORMS and ops.fits_linear_layernorm(o, mlp.fc1.weight)
+    if fold2 and ops.fits_linear_stats(o, attn.proj.weight):
+        q1, rec2 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev, stats_eps=n2.eps)
+    else:
+        q1 = ops.linear(o, attn.proj.weight, attn.proj.bias, residual=comp, rows_dev=rows_dev)
+        rec2 = ops.layernorm_stats(q1, n2.eps, rows_dev=rows_dev) if fold2 else None
 
-    if FOLD_NORMS and ops.fits_linear_layernorm(q1, mlp.fc1.weight):
-        rec2 = ops.layernorm_stats(q1, n2.eps, rows_dev=rows_dev)
+    if fold2:
         hid = ops.linear_layernorm(q1, rec2, mlp.fc1.weight, mlp.fc1.bias, n2.weight, n2.bias, act="gelu",
                                    rows_dev=rows_dev)
     else:

@@ -298,8 +298,15 @@ def packed_weight(weight):
     return packed
 
 
-def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=None):
-    """out = act(a @ weight.T + bias) + residual; a [..., K] (last dim contiguous), weight [N, K]."""
+def fits_linear_stats(a, weight):
+    """Whether `linear(..., stats_eps=...)` has a kernel for these operands (bf16, 384 -> 384, 2048 rows or more)."""
+    return fits_linear_layernorm(a, weight) and weight.shape[0] == 384
+
+
+def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=None, stats_eps=None):
+    """out = act(a @ weight.T + bias) + residual; a [..., K] (last dim contiguous), weight [N, K].
+    With `stats_eps` (a LayerNorm's eps; see `fits_linear_stats`) -> (out, statistics records of the rows of out) for a
+    `linear_layernorm` that takes `out` next."""
     _need_gpu(a, weight, bias, residual)
     _check_like(a, weight=weight, bias=bias, residual=residual, out=out)
     K = a.shape[-1]
@@ -326,6 +333,15 @@ def linear(a, weight, bias=None, residual=None, act="none", rows_dev=None, out=N
         if r2.stride(-1) != 1:
             r2 = r2.contiguous()
     packed = packed_weight(weight) if PACK_WEIGHTS and a.dtype == torch.bfloat16 and rows >= 2048 else None
+    if stats_eps is not None:
+        if act != "none" or not fits_linear_stats(a2, weight):
+            raise ValueError("linear: no kernel that writes statistics records for these operands (see fits_linear_stats)")
+        rec = torch.empty((rows, 16), dtype=torch.bfloat16, device=a.device)
+        call("vtdge_linear_stats", ptr(a2), a2.stride(0), ptr(weight), ptr(packed), ptr(bias), ptr(r2),
+             r2.stride(0) if r2 is not None else 0, ptr(o2), o2.stride(0), ptr(rec), float(stats_eps), ptr(rows_dev),
+             rows, N, K, dtype_code(a), stream_ptr(),
+             tag=("linear_stats", bias is not None, residual is not None, rows, N, K, rows_dev is not None))
+        return out, rec
     call("vtdge_linear_prepacked", ptr(a2), a2.stride(0) if rows > 1 else K, ptr(weight), ptr(packed), ptr(bias), ptr(r2),
          (r2.stride(0) if rows > 1 else N) if r2 is not None else 0, ptr(o2), o2.stride(0) if rows > 1 else N,
          ptr(rows_dev), rows, N, K, _lib.ACT_GELU if act == "gelu" else _lib.ACT_NONE, dtype_code(a), stream_ptr(),
