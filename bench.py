@@ -72,7 +72,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         act = 1 if tag[1] == "gelu" else 0
         rows, N, K = tag[4], tag[5], tag[6]
         if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
-            return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}>"
+            return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}, false, false>"
         if dt == "bf16" and K == 1536 and N % 96 == 0 and N // 96 <= 8 and rows >= 2048 and not act:
             return f"linear_ks_kernel<{b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
@@ -80,7 +80,9 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     if name == "vtdge_linear_layernorm":
-        return f"linear_ws_kernel<24, 3, {1 if tag[1] == 'gelu' else 0}, false, false, true>"
+        return f"linear_ws_kernel<24, 3, {1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
+    if name == "vtdge_linear_stats":
+        return f"linear_ws_kernel<24, 3, 0, {b(tag[1])}, {b(tag[2])}, false, true>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_layernorm_stats":
         nv = tag[2] * esz // 16
@@ -135,6 +137,10 @@ def algorithmic_work(name, tag, esz, geo):
         M = L if packed else rows
         # operands once: A, W, the output and, when there is one, the residual
         return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn * (2 if has_res else 1)) * esz
+    if name == "vtdge_linear_stats":
+        _, _, has_res, rows, Nn, K, packed = tag
+        M = L if packed else rows
+        return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn * (2 if has_res else 1)) * esz + 32 * M
     if name == "vtdge_linear_layernorm":
         _, _, rows, Nn, K, packed = tag
         M = L if packed else rows
