@@ -72,7 +72,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         act = 1 if tag[1] == "gelu" else 0
         rows, N, K = tag[4], tag[5], tag[6]
         if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
-            return f"linear_ws_kernel<24, 3, {act}, {b(tag[2])}, {b(tag[3])}, false, false>"
+            return f"linear_ws8_kernel<{act}, {b(tag[2])}, {b(tag[3])}, false, false>"
         if dt == "bf16" and K == 1536 and N % 96 == 0 and N // 96 <= 8 and rows >= 2048 and not act:
             return f"linear_ks_kernel<{b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
@@ -80,9 +80,9 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     if name == "vtdge_linear_layernorm":
-        return f"linear_ws_kernel<24, 3, {1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
+        return f"linear_ws8_kernel<{1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
     if name == "vtdge_linear_stats":
-        return f"linear_ws_kernel<24, 3, 0, {b(tag[1])}, {b(tag[2])}, false, true>"
+        return f"linear_ws8_kernel<0, {b(tag[1])}, {b(tag[2])}, false, true>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_layernorm_stats":
         nv = tag[2] * esz // 16
@@ -394,7 +394,7 @@ def run_isolated_gemm(args, torch):
                        "packed_rows": L},
             "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": 2500.0, "unit": "TFLOP/s",
                          "frac": round(ach / 2500.0, 4),
-                         "kernel": "linear_ws_kernel<24, 3, 0, true, false>" if L >= 2048
+                         "kernel": "linear_ws8_kernel<0, true, false, false, false>" if L >= 2048
                          else "linear_dma_kernel<unsigned short, ...>",
                          "traffic": None},
             "per_n": per_n}

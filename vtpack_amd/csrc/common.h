@@ -73,7 +73,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
-// Statistics record of a row for the Linear that layer-normalises its input on the fly (linear_ws.hip, HAS_LN):
+// Statistics record of a row for the Linear that layer-normalises its input on the fly (linear_ws8.hip, HAS_LN):
 // 16 bf16 values, the A-side operand of one 16-deep MFMA K step.  mean = m1 + m2 + m3 and sigma = sqrt(var + eps)
 // = s1 + s2 are split into bf16 parts; against the column record (-c1, -c2, -c1, -c3, -c2, -c1, b1, b1 | b2, 0, ...)
 // of a column with colsum c = c1 + c2 + c3 and bias b = b1 + b2 the K step yields -mean * c + sigma * b with all

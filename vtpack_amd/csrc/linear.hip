@@ -185,19 +185,18 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
                       void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K, int act,
                       hipStream_t st);
 
-// weight-stationary variant for bf16, K = 384 (linear_ws.hip)
+// weight-stationary variant for bf16, K = 384 (linear_ws8.hip)
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
-int launch_linear_ws(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
-                     int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
-                     hipStream_t st);
-
-int launch_linear_ws_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
-                        const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
-                        hipStream_t st);
-int launch_linear_ws_stats(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
-                           int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows,
-                           void *records, float eps, hipStream_t st);
+int launch_linear_ws8(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
+                      int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
+                      hipStream_t st);
+int launch_linear_ws8_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
+                         const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N,
+                         int act, hipStream_t st);
+int launch_linear_ws8_stats(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias,
+                            const void *res, int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev,
+                            int64_t rows, void *records, float eps, hipStream_t st);
 
 // K-split weight-stationary variant for bf16, K = 1536, narrow N (linear_ks.hip)
 bool linear_ks_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
@@ -212,8 +211,8 @@ using namespace vtdge;
 // ---------------------------------------------------------------------------------------------------------
 // Packed copies of W for the weight-stationary kernels: the 16-byte register images of the MFMA fragments, in the
 // order [column group][wave][fragment][lane], so a wave fills its registers with contiguous 1 KB loads.
-//   layout 1 (K = 384, linear_ws.hip): group = 384 columns; wave w, fragment (j, s), lane (lr, lg) holds
-//            W[384 g + 96 w + 32 j + lr][16 s + 8 lg .. + 7]                       (j < 3, s < 24)
+//   layout 1 (K = 384, linear_ws8.hip): group = 384 columns; wave w, fragment (cb, ks), lane (c16, kg) holds
+//            W[384 g + 48 w + 16 cb + c16][32 ks + 8 kg .. + 7]                    (w < 8, cb < 3, ks < 12)
 //   layout 2 (K = 1536, linear_ks.hip): group = 96 columns; wave w, fragment (cb, ks), lane (c16, kg) holds
 //            W[96 g + 16 cb + c16][384 w + 32 ks + 8 kg .. + 7]                    (cb < 6, ks < 12)
 static int packed_layout(int N, int K, int dtype)
@@ -230,14 +229,16 @@ __global__ __launch_bounds__(256) void linear_prepack_kernel(const bf16_t *__res
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;       // one 16-byte unit each
     if (idx >= (int64_t)N * K / 8) return;
     const int lane = (int)(idx & 63);
-    const int f = (int)((idx >> 6) % 72), gw = (int)((idx >> 6) / 72);
-    const int w = gw & 3, g = gw >> 2;
     int row, k;
     if (layout == 1) {
-        const int j = f / 24, s = f % 24, lr = lane & 31, lg = lane >> 5;
-        row = 384 * g + 96 * w + 32 * j + lr;
-        k = 16 * s + 8 * lg;
+        const int f = (int)((idx >> 6) % 36), gw = (int)((idx >> 6) / 36);
+        const int w = gw & 7, g = gw >> 3;
+        const int cb = f / 12, ks = f % 12, c16 = lane & 15, kg = lane >> 4;
+        row = 384 * g + 48 * w + 16 * cb + c16;
+        k = 32 * ks + 8 * kg;
     } else {
+        const int f = (int)((idx >> 6) % 72), gw = (int)((idx >> 6) / 72);
+        const int w = gw & 3, g = gw >> 2;
         const int cb = f / 12, ks = f % 12, c16 = lane & 15, kg = lane >> 4;
         row = 96 * g + 16 * cb + c16;
         k = 384 * w + 32 * ks + 8 * kg;
@@ -328,8 +329,8 @@ extern "C" int vtdge_linear_layernorm(const void *A, int64_t lda, const void *ro
                VTDGE_ERR_UNSUPPORTED,
                "linear_layernorm: built for bf16, K = 384, N a multiple of 384 (at most 3072) and 2048 rows or more "
                "(rows=%lld N=%d K=%d dtype=%d)", (long long)rows, N, K, dtype);
-    return launch_linear_ws_ln(A, lda, row_records, W_folded, packed, col_records, out, ldo, rows_dev, rows, N, act,
-                               (hipStream_t)stream);
+    return launch_linear_ws8_ln(A, lda, row_records, W_folded, packed, col_records, out, ldo, rows_dev, rows, N, act,
+                                (hipStream_t)stream);
 }
 
 extern "C" int vtdge_linear_stats(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,
@@ -348,8 +349,8 @@ extern "C" int vtdge_linear_stats(const void *A, int64_t lda, const void *W, con
                VTDGE_ERR_UNSUPPORTED,
                "linear_stats: built for bf16, K = 384, N = 384 and 2048 rows or more (rows=%lld N=%d K=%d dtype=%d)",
                (long long)rows, N, K, dtype);
-    return launch_linear_ws_stats(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, out_records,
-                                  records_eps, (hipStream_t)stream);
+    return launch_linear_ws8_stats(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, out_records,
+                                   records_eps, (hipStream_t)stream);
 }
 
 extern "C" int vtdge_linear(const void *A, int64_t lda, const void *W, const void *bias, const void *residual,
@@ -379,7 +380,7 @@ extern "C" int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W,
     if (rows == 0) return VTDGE_OK;
     hipStream_t st = (hipStream_t)stream;
     if (linear_ws_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
-        return launch_linear_ws(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
+        return launch_linear_ws8(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, N, act, st);
     if (linear_ks_applicable(lda, ldr, ldo, rows, N, K, esz, act, bias, residual, out))
         return launch_linear_ks(A, lda, W, packed, bias, residual, ldr, out, ldo, rows_dev, rows, N, st);
     if (linear_dma_applicable(lda, ldr, ldo, N, K, esz, bias, residual, out)) {

@@ -17,7 +17,7 @@
 // end (their readers are done).  Vector-memory operations retire in issue order and every tile issues the same
 // ones in the same order (no load is conditional: tiles past the end are clamped into the matrix and loaded
 // unused), so a wave waits for its own loads of the tile it starts with a constant s_waitcnt vmcnt.
-// Direct loads and MFMAs are issued from inline assembly (see linear_ws.hip for why).
+// Direct loads and MFMAs are issued from inline assembly (the compiler then adds no vmcnt wait of its own before the LDS reads of the fragments, and the stationary fragments stay in the registers they were put in).
 // The last tile of the matrix is moved back to end at row M, so no tile but a lone first one reaches past the end.
 #include "common.h"
 #include <stdlib.h>
