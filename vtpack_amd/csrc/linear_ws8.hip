@@ -190,11 +190,13 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
         }
         issued += NLA * (HAS_RES ? 2 : 1);
         if constexpr (HAS_LN) {
-            // the records of the tile's 32 rows (lane i: half i % 2 of row i / 2): 1 KB, brought by every wave alike
-            // (the same bytes to the same place) so that all waves count the same operations
-            const int gm = clamp_row(m0 + (lane >> 1));
-            dma16(lnrec, (uint32_t)gm * 32u + (lane & 1) * 16u, lds0 + OFF_L + (k % D) * 1024);
-            issued += 1;
+            // the records of the tile's 32 rows (lane i: half i % 2 of row i / 2): 1 KB, one load; the waves take
+            // turns (a wave waits for its own loads of a tile before the tile's barrier, so the barrier covers it)
+            if (w == (k & 7)) {
+                const int gm = clamp_row(m0 + (lane >> 1));
+                dma16(lnrec, (uint32_t)gm * 32u + (lane & 1) * 16u, lds0 + OFF_L + (k % D) * 1024);
+                issued += 1;
+            }
         }
         set_mark(k);
     };
