@@ -8,7 +8,12 @@ key names, so the same weights drive it and the HIP path.
 
 What pins it: the operator-level functions are checked against oracle/dge_oracle.c (itself pinned
 by closed forms, see its header) in tests/test_oracle_pins.py; the dense pieces are torch library
-routines (F.layer_norm, F.linear, F.gelu, F.conv2d, softmax).
+routines (F.layer_norm, F.linear, F.gelu, F.conv2d, softmax).  The compositions are pinned too:
+deit_dge_forward with an all-fine router equals a dense ViT built from F.conv2d, nn.LayerNorm and
+F.scaled_dot_product_attention on the same state dict (also distilled / pre-logits / no class token),
+and block_forward with an extra token and a mixed gate equals a brute-force loop in which every
+token takes the output of the query that covers it (tests/test_deit_host.py); pvt_dge_forward has the
+same pins in tests/test_pvt_host.py.
 """
 import math
 
