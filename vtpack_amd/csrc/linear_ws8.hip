@@ -6,7 +6,9 @@
 // registers, most of them in accumulation registers, which the MFMA reads directly), so the only operand that
 // moves is A.  A streams HBM/L2 -> LDS in 32-row tiles by direct loads (no VGPR staging) into a ring several tiles
 // deep, and every wave multiplies every tile against its own columns:  D = W_strip * A_tile^T, so a lane owns four
-// consecutive output columns of one row per block and stores them as 8 bytes.
+// consecutive output columns of one row per block.  The address unit takes a store of 16 rows x 32 bytes about as
+// long as one of 16 rows x 64 bytes, so the first two column blocks of a row block leave in one store of 16 bytes a
+// lane (the four lanes of a row regroup their halves with two row swaps) and the third in one of 8 bytes.
 //
 // Why two waves per SIMD: a single wave issues at most one vector instruction every other issue cycle (measured:
 // an FMA every ~7.5 clocks from one wave, every ~3.7 from two) and keeps the matrix pipe 64 % busy with back-to-back
@@ -211,6 +213,9 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
     // elements of a half tile.
     float f4[4], sa = 0.f, sq = 0.f;
     uint32_t rw = 0u;
+    u32x2 o0 = {0u, 0u};
+    // byte offset, from the lane's own first column (4 kg), of its 16 bytes of the pair of column blocks 0 and 1
+    const int pair_off = (16 * (kg & 1) + 8 * (kg >> 1) - 4 * kg) * 2;
     auto epi_element = [&](auto rb_tag, auto e_tag, const unsigned char *rtile, unsigned char *orow, int part) {
         constexpr int RB = decltype(rb_tag)::value, E = decltype(e_tag)::value, cb = E / 4, i = E % 4;
         float f = acc[RB][cb][i];
@@ -240,7 +245,20 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
             u32x2 o;
             o.x = pack_bf16x2(f4[0], f4[1]);
             o.y = pack_bf16x2(f4[2], f4[3]);
-            *reinterpret_cast<u32x2 *>(orow + cb * 32) = o;
+            if (cb == 0) {
+                o0 = o;            // waits for its neighbour
+            } else if (cb == 1) {
+                // Column blocks 0 and 1 leave together, 16 bytes a lane: the lanes kg = 1, 3 of a row hand their
+                // half of block 0 to kg = 0, 2 and take those lanes' half of block 1 (rows of 16 lanes swapped
+                // between the two registers), so lane kg holds columns 16 (kg % 2) + 8 (kg / 2) .. + 7 of the 32
+                // and a store instruction covers 64 contiguous bytes of each of its 16 rows instead of 32.
+                const auto sx = __builtin_amdgcn_permlane16_swap(o0.x, o.x, false, false);
+                const auto sy = __builtin_amdgcn_permlane16_swap(o0.y, o.y, false, false);
+                const u32x4 v = {sx[0], sy[0], sx[1], sy[1]};
+                *reinterpret_cast<u32x4 *>(orow + pair_off) = v;
+            } else {
+                *reinterpret_cast<u32x2 *>(orow + cb * 32) = o;
+            }
         }
         if constexpr (HAS_STAT) {
             if (E == 11) {
@@ -327,7 +345,7 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
             }
         }
     };
-    auto count_stores = [&]() { issued += CB; };
+    auto count_stores = [&]() { issued += CB - 1; };      // blocks 0 and 1 in one store, block 2 in another
 
     // HAS_STAT: the records of tile k from the eight waves' sums: wave w merges rows 4w .. 4w+3, lane l < 8 writing
     // half l % 2 of row 4w + l / 2 (128 contiguous bytes per wave)
