@@ -556,6 +556,47 @@ def test_batched_sparse_gemm(dev, dtype, ta, tb):
             assert rel_err(got.float(), want) <= 2 ** -8
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batched_sparse_gemm_tile_edges_and_empty_samples(dev, dtype):
+    """Q K^T and P V with sample lengths around the 64-row tile (0, 1, 63, 64, 65, 129), a key count and a K extent
+    that are multiples of nothing (n = 71: odd rows, a K tail in every stage), against the CPU restatement."""
+    from vtpack_amd import _C
+    h, d, n = 2, 40, 71
+    la = np.array([0, 1, 63, 64, 65, 129, 0, 7], dtype=np.int64)
+    lb = np.full(len(la), n, dtype=np.int64)
+    q, k = randn(91, h, int(la.sum()), d), randn(92, h, int(lb.sum()), d)
+    p, v = randn(93, h, int(la.sum()), n), randn(94, h, int(lb.sum()), d)
+    if dtype == torch.bfloat16:
+        q, k, p, v = bf16_round(q), bf16_round(k), bf16_round(p), bf16_round(v)
+    tol = 1e-5 if dtype == torch.float32 else 2 ** -8
+    got = _C.batched_sparse_gemm_forward(_t(q, dev, dtype), _t(k, dev, dtype), torch.from_numpy(la),
+                                         torch.from_numpy(lb), False, True)
+    assert rel_err(got.float(), orc.sparse_gemm(q, k, la, lb, False, True)) <= tol
+    got = _C.batched_sparse_gemm_forward(_t(p, dev, dtype), _t(v, dev, dtype), torch.from_numpy(la),
+                                         torch.from_numpy(lb), False, False)
+    assert rel_err(got.float(), orc.sparse_gemm(p, v, la, lb, False, False)) <= tol
+    # P^T dO (the transposed-a form of a backward pass): rows of the result are the n keys of every sample
+    do = randn(95, h, int(la.sum()), d)
+    if dtype == torch.bfloat16:
+        do = bf16_round(do)
+    got = _C.batched_sparse_gemm_forward(_t(p, dev, dtype), _t(do, dev, dtype), torch.from_numpy(la),
+                                         torch.from_numpy(la), True, False)
+    want = orc.sparse_gemm(p, do, la, la, True, False)
+    assert tuple(got.shape) == want.shape and rel_err(got.float(), want) <= tol
+
+
+def test_batched_sparse_gemm_many_samples(dev):
+    """More (sample, head) pairs than a grid dimension holds (70 000): one launch, every product right."""
+    from vtpack_amd import _C
+    B, h, d = 35000, 2, 8
+    la = (np.arange(B) % 3).astype(np.int64)                   # 0, 1 or 2 rows a sample
+    lb = np.full(B, 2, dtype=np.int64)
+    a, b = randn(96, h, int(la.sum()), d), randn(97, h, int(lb.sum()), d)
+    got = _C.batched_sparse_gemm_forward(_t(a, dev), _t(b, dev), torch.from_numpy(la), torch.from_numpy(lb), False,
+                                         True)
+    assert rel_err(got, orc.sparse_gemm(a, b, la, lb, False, True)) <= 1e-5
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,Hr,Wr,C,extra", [(5, 4, 4, 384, 1), (3, 8, 8, 192, 1), (4, 3, 5, 64, 0), (2, 4, 4, 768, 2),
                                                (2, 14, 14, 64, 0), (3, 2, 2, 128, 1)])
