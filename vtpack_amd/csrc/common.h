@@ -137,7 +137,8 @@ template <> struct Elem<bf16_t> {
     static constexpr int VEC = 8;
     static __device__ __forceinline__ float load(const bf16_t *p) { return bf16_to_f32(*p); }
     static __device__ __forceinline__ void store(bf16_t *p, float v) { *p = f32_to_bf16(v); }
-    static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+    // the value as stored: the same hardware conversion as pack() (one convert and one shift)
+    static __device__ __forceinline__ float round(float v) { return bf16lo(pack_bf16x2(v, 0.f)); }
     static __device__ __forceinline__ void unpack(const u32x4 &r, float *f)
     {
         f[0] = bf16lo(r.x); f[1] = bf16hi(r.x); f[2] = bf16lo(r.y); f[3] = bf16hi(r.y);

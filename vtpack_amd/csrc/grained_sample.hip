@@ -525,15 +525,21 @@ __global__ __launch_bounds__(256, NIT == 1 ? 8 : 2) void compress_kernel(const T
                 else if (sz == 2) window_sum<T, 2>(base, W, C, sz, acc);
                 else if (sz == 4) window_sum<T, 4>(base, W, C, sz, acc);
                 else window_sum<T, 0>(base, W, C, sz, acc);
-                const float area = (float)(sz * sz);
+                // mean = sum / area.  The areas of the usual windows are powers of two, whose reciprocals are exact:
+                // the product is then the quotient, bit for bit, at a tenth of the instructions
+                if (sz == 2 || sz == 4) {
+                    const float inv = sz == 2 ? 0.25f : 0.0625f;
 #pragma unroll
-                for (int c = 0; c < VEC; c++) acc[c] = acc[c] / area;
-            }
-            *reinterpret_cast<u32x4 *>(out + row * (int64_t)C + v * VEC) = Elem<T>::pack(acc);
-            if constexpr (LN) {
+                    for (int c = 0; c < VEC; c++) acc[c] = acc[c] * inv;
+                } else if (sz != 1) {
+                    const float area = (float)(sz * sz);
 #pragma unroll
-                for (int c = 0; c < VEC; c++) vals[it][c] = Elem<T>::round(acc[c]);
+                    for (int c = 0; c < VEC; c++) acc[c] = acc[c] / area;
+                }
             }
+            const u32x4 packed = Elem<T>::pack(acc);
+            *reinterpret_cast<u32x4 *>(out + row * (int64_t)C + v * VEC) = packed;
+            if constexpr (LN) Elem<T>::unpack(packed, vals[it]);        // the row as stored
         } else if constexpr (LN) {
 #pragma unroll
             for (int c = 0; c < VEC; c++) vals[it][c] = 0.f;
