@@ -521,17 +521,20 @@ __global__ __launch_bounds__(256, NIT == 1 ? 8 : 2) void compress_kernel(const T
 #pragma unroll
                 for (int c = 0; c < VEC; c++) acc[c] = 0.f;
                 const T *base = xb + ((y0 * W + x0 + extra) * (int64_t)C + v * VEC);
-                if (sz == 1) window_sum<T, 1>(base, W, C, sz, acc);
-                else if (sz == 2) window_sum<T, 2>(base, W, C, sz, acc);
-                else if (sz == 4) window_sum<T, 4>(base, W, C, sz, acc);
-                else window_sum<T, 0>(base, W, C, sz, acc);
                 // mean = sum / area.  The areas of the usual windows are powers of two, whose reciprocals are exact:
                 // the product is then the quotient, bit for bit, at a tenth of the instructions
-                if (sz == 2 || sz == 4) {
-                    const float inv = sz == 2 ? 0.25f : 0.0625f;
+                if (sz == 1) {
+                    window_sum<T, 1>(base, W, C, sz, acc);
+                } else if (sz == 2) {
+                    window_sum<T, 2>(base, W, C, sz, acc);
 #pragma unroll
-                    for (int c = 0; c < VEC; c++) acc[c] = acc[c] * inv;
-                } else if (sz != 1) {
+                    for (int c = 0; c < VEC; c++) acc[c] *= 0.25f;
+                } else if (sz == 4) {
+                    window_sum<T, 4>(base, W, C, sz, acc);
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) acc[c] *= 0.0625f;
+                } else {
+                    window_sum<T, 0>(base, W, C, sz, acc);
                     const float area = (float)(sz * sz);
 #pragma unroll
                     for (int c = 0; c < VEC; c++) acc[c] = acc[c] / area;
