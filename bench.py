@@ -77,8 +77,11 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return f"linear_ks_kernel<{b(tag[2])}, {b(tag[3])}>"
         if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
             tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
-            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false>"
+            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
+    if name == "vtdge_patch_embed":           # tag = ("patch_embed", B, S, patch, C)
+        tile = "256, 128, 4, 2, 4" if tag[4] >= 768 else "128, 128, 2, 2, 4"
+        return f"linear_dma_kernel<{T}, {tile}, 0, true, true, 3, false, true>"
     if name == "vtdge_linear_layernorm":
         return f"linear_ws8_kernel<{1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
     if name == "vtdge_linear_stats":
@@ -137,6 +140,11 @@ def algorithmic_work(name, tag, esz, geo):
         M = L if packed else rows
         # operands once: A, W, the output and, when there is one, the residual
         return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn * (2 if has_res else 1)) * esz
+    if name == "vtdge_patch_embed":
+        # images in, tokens out, the weight and the position table once
+        _, Bp, S, patch, Cc = tag
+        rows, K = Bp * (S // patch) ** 2, 3 * patch * patch
+        return "mfma", 2.0 * rows * Cc * K, (rows * K + Cc * K + rows * Cc + (S // patch) ** 2 * Cc) * esz
     if name == "vtdge_linear_stats":
         _, _, has_res, rows, Nn, K, packed = tag
         M = L if packed else rows

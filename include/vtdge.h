@@ -177,6 +177,18 @@ int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void
                            const void *residual, int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev,
                            int64_t rows, int N, int K, int act, int dtype, void *stream);
 
+/* Patch embedding, position embedding included: the stride-P P x P convolution of the reference's PatchEmbed
+ * (nn.Conv2d, vtpack/models/dge/deit_dge.py:141-155) as a Linear over the patches, read straight from the images
+ * (no unfolded copy), with the addition of the position table (x = x + pos_embed, deit_dge.py:277) in its epilogue:
+ *   images [B, Cin, S, S]   weight [C, Cin * P * P] (the convolution's weight, flattened)   bias [C]
+ *   pos_embed [extra + G*G, C], G = S / P   tokens [B, extra + G*G, C]
+ *   tokens[b, extra + gy*G + gx, :] = conv(images)[b, :, gy, gx] + bias + pos_embed[extra + gy*G + gx, :]
+ * in fp32 with one rounding; rows 0 .. extra-1 of every sample (class / distillation tokens) are left untouched.
+ * A patch row must be 16, 32, 64 or 128 bytes (P = 16: both types) and all operands 16-byte aligned, else
+ * VTDGE_ERR_UNSUPPORTED. */
+int vtdge_patch_embed(const void *images, const void *weight, const void *bias, const void *pos_embed, void *tokens,
+                      int B, int Cin, int S, int P, int C, int extra, int dtype, void *stream);
+
 /* LayerNorm folded into the Linear that consumes it: out = act(LayerNorm(A) W^T + bias) computed from the raw rows
  * of A, so that nn.LayerNorm followed by nn.Linear (norm1 -> kv and norm2 -> fc1,
  * vtpack/models/dge/deit_dge.py:127-128 with :73 and :38-44) costs no pass over the rows of its own:

@@ -627,3 +627,45 @@ def test_scatter_back_with_the_next_router(dev, dtype, B, Hr, Wr, C, extra):
     alone, g0, i0 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp)
     assert g0 is None and i0 is None
     assert torch.equal(alone, ops.decompress(q, patches[:L], x, W, extra, add_ref=True, sub=comp))
+
+
+# ------------------------------------------------------------------ patch embedding
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,S,C,extra", [(3, 64, 192, 1), (2, 256, 384, 1), (2, 96, 768, 2), (5, 32, 64, 0)])
+def test_patch_embed(dev, dtype, B, S, C, extra):
+    """The convolution read straight from the images, bias and position embedding added in its epilogue, against
+    nn.functional.conv2d in fp64; in fp32 also bit for bit against the unfolded Linear followed by the addition."""
+    from vtpack_amd import ops
+    P, Cin = 16, 3
+    G = S // P
+    g = torch.Generator().manual_seed(S + C)
+    img = torch.rand(B, Cin, S, S, generator=g).to(dtype).to(dev)
+    w = (torch.randn(C, Cin, P, P, generator=g) * 0.05).to(dtype).to(dev)
+    b = (torch.randn(C, generator=g) * 0.1).to(dtype).to(dev)
+    pos = (torch.randn(1, extra + G * G, C, generator=g) * 0.5).to(dtype).to(dev)
+    assert ops.fits_patch_embed(img, w, b, pos, P)
+    out = torch.full((B, extra + G * G, C), 7.0, dtype=dtype, device=dev)
+    ops.patch_embed(img, w, b, pos, P, extra, out=out)
+    assert bool((out[:, :extra] == 7.0).all())                       # the rows in front are not touched
+    want = torch.nn.functional.conv2d(img.double(), w.double(), b.double(), stride=P).flatten(2).transpose(1, 2)
+    want = want + pos.double()[:, extra:]
+    err = float((out[:, extra:].double() - want).abs().max())
+    assert err <= (1e-5 if dtype == torch.float32 else 2 ** -8) * float(want.abs().max())
+    if dtype == torch.float32:
+        patches = img.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
+        old = ops.linear(patches, w.reshape(C, -1), b).view(B, G * G, C) + pos[:, extra:]
+        assert torch.equal(out[:, extra:], old)
+
+
+def test_patch_embed_refusals(dev):
+    from vtpack_amd import ops
+    img = torch.zeros(2, 3, 64, 64, device=dev)
+    w = torch.zeros(64, 3, 4, 4, device=dev)
+    assert not ops.fits_patch_embed(img.bfloat16(), w.bfloat16(), torch.zeros(64, device=dev).bfloat16(),
+                                    torch.zeros(1, 257, 64, device=dev).bfloat16(), 4)      # 8-byte patch rows
+    with pytest.raises(ValueError):
+        ops.patch_embed(img, torch.zeros(64, 3, 16, 16, device=dev), torch.zeros(64, device=dev),
+                        torch.zeros(1, 99, 64, device=dev), 16, 1)                           # wrong table height
+    with pytest.raises(TypeError):
+        ops.patch_embed(img, torch.zeros(64, 3, 16, 16, device=dev).bfloat16(), torch.zeros(64, device=dev),
+                        torch.zeros(1, 17, 64, device=dev), 16, 1)

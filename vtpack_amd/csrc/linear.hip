@@ -185,6 +185,13 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
                       void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int K, int act,
                       hipStream_t st);
 
+// the patch embedding on the same kernel (linear_dma.hip)
+bool patch_embed_applicable(int P, int S, int Cin, int N, int esz, const void *images, const void *weight,
+                            const void *bias, const void *pos, const void *out);
+template <typename T>
+int launch_patch_embed(const void *images, const void *W, const void *bias, const void *pos, void *out, int B, int Cin,
+                       int S, int P, int N, int extra, hipStream_t st);
+
 // weight-stationary variant for bf16, K = 384 (linear_ws8.hip)
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
@@ -391,4 +398,21 @@ extern "C" int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W,
     if (dtype == VTDGE_F32)
         return launch_linear<float>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
     return launch_linear<bf16_t>(A, lda, W, bias, residual, ldr, out, ldo, rows_dev, rows, N, K, act, st);
+}
+
+extern "C" int vtdge_patch_embed(const void *images, const void *weight, const void *bias, const void *pos_embed,
+                                 void *tokens, int B, int Cin, int S, int P, int C, int extra, int dtype, void *stream)
+{
+    VT_REQUIRE(images && weight && tokens, VTDGE_ERR_ARG, "patch_embed: NULL operand");
+    VT_REQUIRE(dtype == VTDGE_F32 || dtype == VTDGE_BF16, VTDGE_ERR_ARG, "patch_embed: unknown dtype %d", dtype);
+    VT_REQUIRE(B > 0 && Cin > 0 && S > 0 && P > 0 && C > 0 && extra >= 0, VTDGE_ERR_ARG, "patch_embed: bad sizes");
+    const int esz = dtype == VTDGE_F32 ? 4 : 2;
+    VT_REQUIRE(patch_embed_applicable(P, S, Cin, C, esz, images, weight, bias, pos_embed, tokens), VTDGE_ERR_UNSUPPORTED,
+               "patch_embed: no kernel for patch %d, image %d, %d channels, width %d (or bias / position table missing, "
+               "or an operand not 16-byte aligned)", P, S, Cin, C);
+    VT_REQUIRE((int64_t)B * Cin * S * S < (1ll << 40), VTDGE_ERR_UNSUPPORTED, "patch_embed: batch too large");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_F32)
+        return launch_patch_embed<float>(images, weight, bias, pos_embed, tokens, B, Cin, S, P, C, extra, st);
+    return launch_patch_embed<bf16_t>(images, weight, bias, pos_embed, tokens, B, Cin, S, P, C, extra, st);
 }

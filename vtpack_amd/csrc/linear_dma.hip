@@ -61,12 +61,24 @@ template <> __device__ __forceinline__ float gelu_fn<bf16_t>(float v)
 // trims each XCD's list.
 // NSTAGE = depth of the operand ring (3, or 2 for tiles whose stages are too large for three); LATE = fetch bias and
 // residual in the epilogue itself instead of during the last stage (large wave tiles have no registers to park them).
+//
+// PATCH: the kernel is a patch embedding (a convolution whose stride is its kernel size, as a Linear over the
+// patches).  A is the image batch [B, Cin, S, S] itself: row (b, gy, gx) of the product is patch (gy, gx) of image b
+// and its K index runs over (channel, row of the patch, pixel), so a 128-byte K slab of a row is a few consecutive
+// pixel rows of one channel of the patch and the loader waves fetch them straight from the image - nothing but
+// their per-lane source addresses differs from the plain kernel, no unfolded copy of the images exists.  The output
+// row goes to token `extra + gy G + gx` of sample b in [B, extra + G G, N], and the residual is row
+// `extra + gy G + gx` of one [extra + G G, N] table for every sample (the position embedding).
+struct PatchGeom {
+    int P, S, G, Cin, extra;     // patch edge, image edge, patches per edge, input channels, tokens in front
+};
+
 template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HAS_BIAS, bool HAS_RES, int NSTAGE = 3,
-          bool LATE = false>
+          bool LATE = false, bool PATCH = false>
 __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
     const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, const T *__restrict__ bias,
     const T *__restrict__ res, int64_t ldr, T *__restrict__ out, int64_t ldo, const int64_t *__restrict__ rows_dev,
-    int64_t rows, int N, int K)
+    int64_t rows, int N, int K, PatchGeom pg)
 {
     constexpr int ESZ = sizeof(T);
     static_assert(NSTAGE == 2 || NSTAGE == 3, "ring depth");
@@ -110,7 +122,16 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                 if (r < BM) {
                     int64_t gm = m0 + r;
                     gm = gm < M ? gm : M - 1;
-                    src[i] = reinterpret_cast<const unsigned char *>(A + gm * lda) + chunk * 16;
+                    if constexpr (PATCH) {
+                        // patch (b, gy, gx); the chunk is pixels `cc` of patch row `cr` of the slab's first rows
+                        const int g2 = pg.G * pg.G, cpr = pg.P * ESZ / 16;      // chunks per patch row
+                        const int b = (int)(gm / g2), t = (int)(gm % g2), gy = t / pg.G, gx = t % pg.G;
+                        const int cr = chunk / cpr, cc = chunk % cpr;
+                        src[i] = reinterpret_cast<const unsigned char *>(
+                                     A + ((int64_t)b * pg.Cin * pg.S + gy * pg.P + cr) * pg.S + gx * pg.P) + cc * 16;
+                    } else {
+                        src[i] = reinterpret_cast<const unsigned char *>(A + gm * lda) + chunk * 16;
+                    }
                 } else {
                     int gn = n0 + r - BM;
                     gn = gn < N ? gn : N - 1;
@@ -122,8 +143,17 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
         set_tile(0);
         auto issue_next = [&]() {
             unsigned char *dst = smem + (issued % NSTAGE) * STAGE + lw * NLW * 1024;
+            int64_t a_off = (int64_t)it_kt * DKB;
+            if constexpr (PATCH) {
+                // slab it_kt of a patch: its channel and its first row in the patch
+                const int rps = DKB / (pg.P * ESZ), spc = pg.P / rps;          // rows per slab, slabs per channel
+                a_off = ((int64_t)(it_kt / spc) * pg.S + (it_kt % spc) * rps) * pg.S * ESZ;
+            }
 #pragma unroll
-            for (int i = 0; i < NLW; i++) VT_GLOBAL_TO_LDS(src[i] + (int64_t)it_kt * DKB, dst + i * 1024);
+            for (int i = 0; i < NLW; i++) {
+                const bool a_rows = (lw * NLW + i) * 8 < BM;
+                VT_GLOBAL_TO_LDS(src[i] + (a_rows ? a_off : (int64_t)it_kt * DKB), dst + i * 1024);
+            }
             issued++;
             if (++it_kt == nk) {
                 it_kt = 0;
@@ -145,6 +175,15 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
     }
 
     // ---- MFMA side
+    // where row `row` of the product is stored and which row of the residual it takes
+    auto out_row = [&](int64_t row) -> int64_t {
+        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return row + (row / g2 + 1) * pg.extra; }
+        else return row;
+    };
+    auto res_row = [&](int64_t row) -> int64_t {
+        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return row % g2 + pg.extra; }
+        else return row;
+    };
     const int wm = wid / WGN, wn = wid % WGN;
     const int lr = lane & 31, lg = lane >> 5;
     const int sw = (lr >> 1) & 7;
@@ -190,7 +229,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                         rraw[i][j][q] = z;
                         if constexpr (HAS_RES)
                             if (row < M && col < N)
-                                rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + row * ldr + col);
+                                rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + res_row(row) * ldr + col);
                     }
                 }
         }
@@ -243,7 +282,8 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                         if constexpr (HAS_BIAS)
                             if (col < N) braw[j][q] = *reinterpret_cast<const u32x4 *>(bias + col);
                         if constexpr (HAS_RES)
-                            if (row < M && col < N) rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + row * ldr + col);
+                            if (row < M && col < N)
+                                rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + res_row(row) * ldr + col);
                     }
                     if constexpr (HAS_BIAS) {
                         float bv[EPL];
@@ -261,7 +301,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
 #pragma unroll
                         for (int e = 0; e < EPL; e++) f[e] += rv[e];
                     }
-                    if (row < M && col < N) *reinterpret_cast<u32x4 *>(out + row * ldo + col) = Elem<T>::pack(f);
+                    if (row < M && col < N) *reinterpret_cast<u32x4 *>(out + out_row(row) * ldo + col) = Elem<T>::pack(f);
                 }
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
@@ -276,8 +316,8 @@ struct LinArgs {
     void *out; int64_t ldo; const int64_t *rows_dev; int64_t rows; int N; int K; int act; hipStream_t st;
 };
 
-template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HB, bool HR>
-static int go(const LinArgs &a)
+template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HB, bool HR, bool PATCH = false>
+static int go(const LinArgs &a, const PatchGeom &pg = PatchGeom{0, 0, 0, 0, 0})
 {
     constexpr int NW = WGM * WGN + NWP;
     constexpr int NSTAGE = (size_t)3 * (BM + BN) * DKB <= 160 * 1024 ? 3 : 2;
@@ -285,7 +325,7 @@ static int go(const LinArgs &a)
     constexpr size_t lds = (size_t)NSTAGE * (BM + BN) * DKB;
     static_assert(lds <= 160 * 1024, "LDS budget");
     constexpr int WGS_PER_CU = lds <= 80 * 1024 ? 2 : 1;
-    auto kern = linear_dma_kernel<T, BM, BN, WGM, WGN, NWP, ACT, HB, HR, NSTAGE, LATE>;
+    auto kern = linear_dma_kernel<T, BM, BN, WGM, WGN, NWP, ACT, HB, HR, NSTAGE, LATE, PATCH>;
     VT_RESERVE_LDS(kern, lds, "linear");
     // persistent grid: what fits on the 256 CUs at once, but never more workgroups than tiles per XCD
     const int64_t tiles_per_xcd = ceil_div(ceil_div(a.rows, BM), 8) * ceil_div(a.N, BN);
@@ -293,7 +333,7 @@ static int go(const LinArgs &a)
     if (wgs_per_xcd > tiles_per_xcd) wgs_per_xcd = tiles_per_xcd;
     dim3 grid((unsigned)(wgs_per_xcd * 8)), block(NW * 64);
     kern<<<grid, block, lds, a.st>>>((const T *)a.A, a.lda, (const T *)a.W, (const T *)a.bias, (const T *)a.res,
-                                     a.ldr, (T *)a.out, a.ldo, a.rows_dev, a.rows, a.N, a.K);
+                                     a.ldr, (T *)a.out, a.ldo, a.rows_dev, a.rows, a.N, a.K, pg);
     return check_launch("linear");
 }
 
@@ -333,6 +373,32 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
     if (N >= 768) return pick_epilogue<T, 256, 128, 4, 2, 4>(a);
     return pick_epilogue<T, 128, 128, 2, 2, 4>(a);
 }
+
+// The patch embedding: images [B, Cin, S, S] -> tokens [B, extra + G G, N] rows extra.., = conv + bias + pos.
+bool patch_embed_applicable(int P, int S, int Cin, int N, int esz, const void *images, const void *weight,
+                            const void *bias, const void *pos, const void *out)
+{
+    const int row = P * esz;                 // bytes of a patch row
+    return P > 0 && S % P == 0 && row % 16 == 0 && DKB % row == 0 && P % (DKB / row) == 0 &&
+           ((int64_t)S * esz) % 16 == 0 && N % (16 / esz) == 0 && bias != nullptr && pos != nullptr &&
+           (((uintptr_t)images | (uintptr_t)weight | (uintptr_t)bias | (uintptr_t)pos | (uintptr_t)out) & 15) == 0;
+}
+
+template <typename T>
+int launch_patch_embed(const void *images, const void *W, const void *bias, const void *pos, void *out, int B, int Cin,
+                       int S, int P, int N, int extra, hipStream_t st)
+{
+    const int G = S / P;
+    const PatchGeom pg{P, S, G, Cin, extra};
+    LinArgs a{images, 0, W, bias, pos, N, out, N, nullptr, (int64_t)B * G * G, N, Cin * P * P, VTDGE_ACT_NONE, st};
+    if (N >= 768) return go<T, 256, 128, 4, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
+    return go<T, 128, 128, 2, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
+}
+
+template int launch_patch_embed<float>(const void *, const void *, const void *, const void *, void *, int, int, int,
+                                       int, int, int, hipStream_t);
+template int launch_patch_embed<bf16_t>(const void *, const void *, const void *, const void *, void *, int, int, int,
+                                        int, int, int, hipStream_t);
 
 template int launch_linear_dma<float>(const void *, int64_t, const void *, const void *, const void *, int64_t, void *,
                                       int64_t, const int64_t *, int64_t, int, int, int, hipStream_t);

@@ -35,6 +35,9 @@ FUSE_NEXT_ROUTER = True
 # takes the raw rows and a 32-byte statistics record per row, so no normalised copy of the tokens is written or read.
 # Taken where the weight-stationary kernel applies (bf16, 384 channels, 2048 rows or more, no spatial reduction).
 FOLD_NORMS = True
+# The patch embedding read straight from the images, position embedding added in its epilogue (`vtdge_patch_embed`),
+# instead of an unfolded copy of the images, a Linear, a copy into the token tensor and an addition.
+FUSE_PATCH_EMBED = True
 
 
 def _side_stream(device, slot=0):
@@ -239,9 +242,10 @@ def _run_blocks(blocks, x, H, W):
 def model_forward(model, images):
     """images [B, 3, S, S] -> logits for a `VisionTransformer` in eval mode, dense pieces included.
 
-    The patch embedding (a stride-16 16x16 convolution, i.e. a Linear over unfolded patches), the final
-    LayerNorm (only the class-token rows are needed) and the classifier run on the same libvtdge kernels;
-    torch contributes only the unfold / concat / add copy kernels.  vtpack/models/dge/deit_dge.py:267-299.
+    The patch embedding (a stride-16 16x16 convolution, i.e. a Linear over the patches, read straight from the
+    images, with the position embedding added on the way out), the final LayerNorm (only the class-token rows are
+    needed) and the classifier run on the same libvtdge kernels; torch contributes only the few rows of the class
+    tokens.  vtpack/models/dge/deit_dge.py:267-299.
     """
     pe = model.patch_embed
     B, Cin, S, _ = images.shape
@@ -250,15 +254,21 @@ def model_forward(model, images):
     P = pe.patch_size[0]
     G = S // P
     C = model.embed_dim
-    patches = images.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
     front = [t for t in (model.cls_token, getattr(model, "dist_token", None)) if t is not None]
     extra = len(front)
-    x = torch.empty((B, extra + G * G, C), dtype=images.dtype, device=images.device)
-    tok = ops.linear(patches, pe.proj.weight.reshape(C, Cin * P * P), pe.proj.bias)
-    x[:, extra:, :] = tok.view(B, G * G, C)
-    for e, t in enumerate(front):
-        x[:, e:e + 1, :] = t
-    x += model.pos_embed
+    if FUSE_PATCH_EMBED and ops.fits_patch_embed(images, pe.proj.weight, pe.proj.bias, model.pos_embed, P):
+        # the convolution reads the images in place and adds the position embedding on its way out
+        x = ops.patch_embed(images, pe.proj.weight, pe.proj.bias, model.pos_embed, P, extra)
+        for e, t in enumerate(front):
+            x[:, e:e + 1, :] = t + model.pos_embed[:, e:e + 1, :]
+    else:
+        patches = images.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
+        x = torch.empty((B, extra + G * G, C), dtype=images.dtype, device=images.device)
+        tok = ops.linear(patches, pe.proj.weight.reshape(C, Cin * P * P), pe.proj.bias)
+        x[:, extra:, :] = tok.view(B, G * G, C)
+        for e, t in enumerate(front):
+            x[:, e:e + 1, :] = t
+        x += model.pos_embed
     x = _run_blocks(list(model.blocks), x, G, G)
     nrm = model.norm
 

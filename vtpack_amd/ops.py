@@ -408,6 +408,48 @@ def folded_weight(weight, bias, ln_weight, ln_bias):
     return value
 
 
+def fits_patch_embed(images, weight, bias, pos_embed, patch):
+    """Whether `patch_embed` has a kernel: a patch row of 16, 32, 64 or 128 bytes (patch 16 in both types), square
+    images whose edge is a multiple of the patch, bias and position table present."""
+    if images.dim() != 4 or images.shape[2] != images.shape[3] or bias is None or pos_embed is None:
+        return False
+    esz = images.element_size()
+    row = patch * esz
+    S = images.shape[2]
+    return (images.dtype in (torch.float32, torch.bfloat16) and patch > 0 and S % patch == 0 and row % 16 == 0
+            and 128 % row == 0 and patch % (128 // row) == 0 and (S * esz) % 16 == 0
+            and weight.shape[0] % (16 // esz) == 0)
+
+
+def patch_embed(images, weight, bias, pos_embed, patch, extra, out=None):
+    """tokens [B, extra + G*G, C]: rows extra.. of every sample = the stride-`patch` convolution of `images`
+    [B, Cin, S, S] with `weight` [C, Cin, patch, patch] (or flattened) + bias + pos_embed[extra..]; rows before them
+    are left as they are (uninitialised in a fresh tensor).  Replaces PatchEmbed's Conv2d and the addition of the
+    position embedding (vtpack/models/dge/deit_dge.py:141-155, :277) without an unfolded copy of the images."""
+    _need_gpu(images, weight, bias, pos_embed)
+    _check_like(images, weight=weight, bias=bias, pos_embed=pos_embed, out=out)
+    if not fits_patch_embed(images, weight, bias, pos_embed, patch):
+        raise ValueError("patch_embed: no kernel for these operands (see fits_patch_embed)")
+    B, Cin, S, _ = images.shape
+    G = S // patch
+    C = weight.shape[0]
+    w2 = _contig(weight.reshape(C, -1))
+    if w2.shape[1] != Cin * patch * patch:
+        raise ValueError(f"weight {tuple(weight.shape)} does not take {Cin} x {patch} x {patch} patches")
+    _check_vector("bias", bias, C)
+    pos = _contig(pos_embed.reshape(-1, C))
+    if pos.shape[0] != extra + G * G:
+        raise ValueError(f"pos_embed holds {pos.shape[0]} rows, the tokens {extra + G * G}")
+    images = _contig(images)
+    if out is None:
+        out = torch.empty((B, extra + G * G, C), dtype=images.dtype, device=images.device)
+    elif tuple(out.shape) != (B, extra + G * G, C) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous tensor of shape {(B, extra + G * G, C)}")
+    call("vtdge_patch_embed", ptr(images), ptr(w2), ptr(_contig(bias)), ptr(pos), ptr(out), B, Cin, S, patch, C, extra,
+         dtype_code(images), stream_ptr(), tag=("patch_embed", B, S, patch, C))
+    return out
+
+
 def linear_layernorm(a, records, weight, bias, ln_weight, ln_bias, act="none", rows_dev=None, out=None):
     """out = act(LayerNorm(a) @ weight.T + bias) from the raw rows a [..., 384] and their statistics records (from
     `layernorm_stats` or from the kernel that produced the rows): no normalised copy of `a` is written or read.
