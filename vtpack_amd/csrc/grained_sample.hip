@@ -781,6 +781,22 @@ __global__ __launch_bounds__(256) void decompress_ln_kernel(const T *__restrict_
 // The group of a sample's first region also scatters the sample's extra tokens.
 // Statistics record of one stored row from the group's sums of (x - pivot) and (x - pivot)^2, the pivot being a value
 // of the row itself (no cancellation however far the row's mean is from zero).  Values are wave-uniform.
+// Lane exchanges of the record sums below: the value of the lane whose number differs in one bit.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// v summed over the lanes that differ in bits 2..5 of the lane number (16 of them), returned in each of them
+__device__ __forceinline__ float sum_over_lane_bits_2_to_5(float v)
+{
+    v += dpp_move<0x141>(dpp_move<0x1B>(v));      // lane ^ 4: the quad reversed, then the half row mirrored
+    v += dpp_move<0x128>(v);                      // lane ^ 8: the row rotated by eight
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);        // lane ^ 16: odd rows swapped with even rows
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);     // lane ^ 32: the halves swapped
+}
+
 __device__ __forceinline__ void row_record(float pivot, float s1, float s2, int C, float eps, u32x4 &lo, u32x4 &hi)
 {
     const float m = s1 / (float)C;
@@ -862,17 +878,30 @@ __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T
             }
         }
         if constexpr (STAT) {
-            wave_sum_n<8>(st);
-            // the four records are 128 contiguous bytes: lane l < 8 writes half l % 2 of token l / 2
-            u32x4 mine = {0u, 0u, 0u, 0u};
+            // The eight sums (two per token) are added up over the wave so that each lane ends with the pair of ONE
+            // token: lanes exchange halves of what they hold with lane ^ 1 (even lanes keep tokens 0 and 1, odd ones
+            // 2 and 3), then with lane ^ 2, and the remaining pair is summed over the other four lane bits.  Lane l
+            // then holds token 2 (l % 2) + (l / 2) % 2, works out that token's record - the four records are made side
+            // by side in different lanes, not one after the other in all of them - and lanes 0..7 write the 128
+            // contiguous bytes: half (l / 4) % 2 of their token.
+            const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
+            float r4[4];
 #pragma unroll
-            for (int dx = 0; dx < 4; dx++) {
-                u32x4 lo, hi;
-                row_record(pivot[dx], st[2 * dx], st[2 * dx + 1], C, eps, lo, hi);
-                if (lane == 2 * dx) mine = lo;
-                if (lane == 2 * dx + 1) mine = hi;
+            for (int i = 0; i < 4; i++) {
+                const float keep = b0 ? st[4 + i] : st[i], send = b0 ? st[i] : st[4 + i];
+                r4[i] = keep + dpp_move<0xB1>(send);                 // lane ^ 1
             }
-            if (lane < 8) rec[(int64_t)dy * W * 2 + lane] = mine;
+            float tot[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const float keep = b1 ? r4[2 + i] : r4[i], send = b1 ? r4[i] : r4[2 + i];
+                tot[i] = sum_over_lane_bits_2_to_5(keep + dpp_move<0x4E>(send));      // lane ^ 2, then the rest
+            }
+            const float pv = b0 ? (b1 ? pivot[3] : pivot[2]) : (b1 ? pivot[1] : pivot[0]);
+            u32x4 lo, hi;
+            row_record(pv, tot[0], tot[1], C, eps, lo, hi);
+            const int tok = 2 * (lane & 1) + ((lane >> 1) & 1), half = (lane >> 2) & 1;
+            if (lane < 8) rec[((int64_t)dy * W + tok) * 2 + half] = half ? hi : lo;
         }
     }
 }
