@@ -125,7 +125,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                     if constexpr (PATCH) {
                         // patch (b, gy, gx); the chunk is pixels `cc` of patch row `cr` of the slab's first rows
                         const int g2 = pg.G * pg.G, cpr = pg.P * ESZ / 16;      // chunks per patch row
-                        const int b = (int)(gm / g2), t = (int)(gm % g2), gy = t / pg.G, gx = t % pg.G;
+                        const int gmi = (int)gm, b = gmi / g2, t = gmi - b * g2, gy = t / pg.G, gx = t - gy * pg.G;
                         const int cr = chunk / cpr, cc = chunk % cpr;
                         src[i] = reinterpret_cast<const unsigned char *>(
                                      A + ((int64_t)b * pg.Cin * pg.S + gy * pg.P + cr) * pg.S + gx * pg.P) + cc * 16;
@@ -176,12 +176,13 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
 
     // ---- MFMA side
     // where row `row` of the product is stored and which row of the residual it takes
+    // (32-bit arithmetic: the patch count of a batch fits, and a 64-bit division costs a hundred instructions)
     auto out_row = [&](int64_t row) -> int64_t {
-        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return row + (row / g2 + 1) * pg.extra; }
+        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return row + ((int)row / g2 + 1) * pg.extra; }
         else return row;
     };
     auto res_row = [&](int64_t row) -> int64_t {
-        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return row % g2 + pg.extra; }
+        if constexpr (PATCH) { const int g2 = pg.G * pg.G; return (int)row % g2 + pg.extra; }
         else return row;
     };
     const int wm = wid / WGN, wn = wid % WGN;
@@ -254,6 +255,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
 #pragma unroll
         for (int i = 0; i < IM; i++) {
             const int64_t row = m0 + wm * TM + i * 32 + lr;
+            const int64_t orow = out_row(row), rrow = res_row(row);
 #pragma unroll
             for (int j = 0; j < JN; j++) {
 #pragma unroll
@@ -283,7 +285,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                             if (col < N) braw[j][q] = *reinterpret_cast<const u32x4 *>(bias + col);
                         if constexpr (HAS_RES)
                             if (row < M && col < N)
-                                rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + res_row(row) * ldr + col);
+                                rraw[i][j][q] = *reinterpret_cast<const u32x4 *>(res + rrow * ldr + col);
                     }
                     if constexpr (HAS_BIAS) {
                         float bv[EPL];
@@ -301,7 +303,7 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
 #pragma unroll
                         for (int e = 0; e < EPL; e++) f[e] += rv[e];
                     }
-                    if (row < M && col < N) *reinterpret_cast<u32x4 *>(out + out_row(row) * ldo + col) = Elem<T>::pack(f);
+                    if (row < M && col < N) *reinterpret_cast<u32x4 *>(out + orow * ldo + col) = Elem<T>::pack(f);
                 }
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
