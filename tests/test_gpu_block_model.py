@@ -153,6 +153,34 @@ def test_deit_tiny_fp32_model(dev, fused):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_model_with_and_without_fused_patch_embedding(dev, dtype):
+    """The patch embedding read straight from the images (position embedding in its epilogue) against the unfolded
+    copy + Linear + addition: the same logits bit for bit in fp32, the same routing and logits within two bf16
+    steps in bf16 (one rounding of the tokens instead of two)."""
+    from vtpack_amd import engine
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_tiny_patch16_256", dev, dtype)
+    img = synthetic_images(4, 256, seed=2).to(dev).to(dtype)
+    assert engine.FUSE_PATCH_EMBED
+    with torch.no_grad():
+        got = m(img)
+        tok = m.blocks[0].dge.states["input"].clone()
+        engine.FUSE_PATCH_EMBED = False
+        try:
+            ref = m(img)
+            tok_ref = m.blocks[0].dge.states["input"]
+        finally:
+            engine.FUSE_PATCH_EMBED = True
+    if dtype == torch.float32:
+        assert torch.equal(tok, tok_ref) and torch.equal(got, ref)
+    else:
+        # the tokens differ by the one rounding saved; a routing decision on a near tie may follow them, so the
+        # logits get the model-level bf16 bound
+        assert abs_err(tok.float(), tok_ref.float()) <= 2.0 ** -7 * float(tok_ref.float().abs().max())
+        assert abs_err(got.float(), ref.float()) <= 2e-2 * max(1.0, float(ref.float().abs().max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_model_with_fused_next_layernorm(dev, dtype):
     """The scatter-back that also writes the next block's first LayerNorm is an option of the fused path: with it
     the model gives the same gate choices and, the two LayerNorm kernels being one arithmetic, the same logits."""
