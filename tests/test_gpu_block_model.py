@@ -328,3 +328,35 @@ def test_states_of_fused_and_layer_mode_agree(dev):
     assert torch.equal(st_f["comp"], st_l["comp"])
     assert st_f["size"] == st_l["size"] and st_f["num_extra_tokens"] == st_l["num_extra_tokens"] == 1
     assert rel_err(out_f, out_l) <= FP32_REL
+
+
+def test_forward_captured_in_a_graph_follows_its_input(dev):
+    """The whole forward holds no synchronisation and no host-side length (every packed kernel reads the live row
+    count from device memory), so it can be captured once in a HIP graph and replayed on new images written into
+    the captured input buffer: the router then takes other decisions and the row counts change inside the graph.
+    Every replay must give, bit for bit, what the eager forward gives for the same images - with eager work and
+    synchronisations of the program between the replays, and the two streams of a block inside the capture."""
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_small_patch16_256", dev, torch.bfloat16)
+    static_in = synthetic_images(8, 256, seed=11, dtype=torch.bfloat16).to(dev)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):           # warm-up off the default stream, as capture requires
+            m(static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            static_out = m(static_in)
+        counts = []
+        for seed in (11, 12, 13, 11):
+            img = synthetic_images(8, 256, seed=seed, dtype=torch.bfloat16).to(dev)
+            eager = m(img)
+            counts.append(int(m.blocks[3].dge.states["batches_device"].sum()))
+            torch.cuda.synchronize()
+            static_in.copy_(img)
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, eager), f"replay on the images of seed {seed} differs from the eager forward"
+    assert len(set(counts[:3])) > 1, "the inputs were meant to change the number of queries"
