@@ -83,6 +83,11 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         big = tag[4] >= 768 or -(-(tag[1] * (tag[2] // tag[3]) ** 2) // 256) * -(-tag[4] // 128) >= 512
         tile = "256, 128, 4, 2, 4" if big else "128, 128, 2, 2, 4"
         return f"linear_dma_kernel<{T}, {tile}, 0, true, true, 3, false, true>"
+    if name == "vtdge_patch_linear":          # tag = ("patch_linear", B, H, W, C, k, N)
+        rows = tag[1] * (tag[2] // tag[5]) * (tag[3] // tag[5])
+        big = tag[6] >= 768 or -(-rows // 256) * -(-tag[6] // 128) >= 512
+        tile = "256, 128, 4, 2, 4" if big else "128, 128, 2, 2, 4"
+        return f"linear_dma_kernel<{T}, {tile}, 0, true, false, 3, false, true>"
     if name == "vtdge_linear_layernorm":
         return f"linear_ws8_kernel<{1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
     if name == "vtdge_linear_stats":
@@ -146,6 +151,11 @@ def algorithmic_work(name, tag, esz, geo):
         _, Bp, S, patch, Cc = tag
         rows, K = Bp * (S // patch) ** 2, 3 * patch * patch
         return "mfma", 2.0 * rows * Cc * K, (rows * K + Cc * K + rows * Cc + (S // patch) ** 2 * Cc) * esz
+    if name == "vtdge_patch_linear":
+        # the tokens in, the weight once, the rows out
+        _, Bp, Hp, Wp, Cp, kp, Np = tag
+        rows, K = Bp * (Hp // kp) * (Wp // kp), kp * kp * Cp
+        return "mfma", 2.0 * rows * Np * K, (rows * K + Np * K + rows * Np) * esz
     if name == "vtdge_linear_stats":
         _, _, has_res, rows, Nn, K, packed = tag
         M = L if packed else rows

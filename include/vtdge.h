@@ -189,6 +189,19 @@ int vtdge_linear_prepacked(const void *A, int64_t lda, const void *W, const void
 int vtdge_patch_embed(const void *images, const void *weight, const void *bias, const void *pos_embed, void *tokens,
                       int B, int Cin, int S, int P, int C, int extra, int dtype, void *stream);
 
+/* A stride-P P x P convolution over a channels-last token grid, as a Linear over the P x P blocks of tokens read
+ * straight from the grid (no gathered copy): the spatial reduction in front of the key/value projection
+ * (nn.Conv2d(dim, dim, sr_ratio, sr_ratio), vtpack/models/dge/pvt_dge.py:62, :81-83) and the patch embedding of the
+ * later stages (nn.Conv2d(in_chans, embed_dim, patch_size, patch_size), pvt_dge.py:164, :175), whose input here stays
+ * [B, H*W, C] tokens instead of going back to [B, C, H, W]:
+ *   tokens [B, H*W, C]   weight [N, P*P*C], the convolution's weight in (kh, kw, c) order   bias [N]
+ *   out [B*(H/P)*(W/P), N]:  out[(b, gy, gx), :] = sum over (dy, dx, c) of
+ *        tokens[b, (gy*P + dy)*W + gx*P + dx, c] * weight[:, (dy*P + dx)*C + c]  + bias,   fp32 sums, one rounding.
+ * C values must fill whole 128-byte pieces (C % 64 == 0 for bf16, % 32 for fp32), H and W be multiples of P and all
+ * operands 16-byte aligned, else VTDGE_ERR_UNSUPPORTED. */
+int vtdge_patch_linear(const void *tokens, const void *weight, const void *bias, void *out, int B, int H, int W, int C,
+                       int P, int N, int dtype, void *stream);
+
 /* LayerNorm folded into the Linear that consumes it: out = act(LayerNorm(A) W^T + bias) computed from the raw rows
  * of A, so that nn.LayerNorm followed by nn.Linear (norm1 -> kv and norm2 -> fc1,
  * vtpack/models/dge/deit_dge.py:127-128 with :73 and :38-44) costs no pass over the rows of its own:

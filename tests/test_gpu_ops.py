@@ -6,6 +6,7 @@ floating point within the tolerances stated in tests/util.py.
 import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import dge_oracle as orc
 from oracle import torch_ref
@@ -669,3 +670,40 @@ def test_patch_embed_refusals(dev):
     with pytest.raises(TypeError):
         ops.patch_embed(img, torch.zeros(64, 3, 16, 16, device=dev).bfloat16(), torch.zeros(64, device=dev),
                         torch.zeros(1, 17, 64, device=dev), 16, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,W,C,k,N", [(3, 8, 8, 64, 2, 128), (2, 16, 24, 128, 4, 128), (2, 16, 16, 64, 8, 64),
+                                         (5, 14, 14, 320, 2, 512), (70, 28, 28, 128, 2, 320)])
+def test_patch_linear(dev, dtype, B, H, W, C, k, N):
+    """The strided convolution over a channels-last token grid read in place (vtdge_patch_linear) against
+    F.conv2d in fp64 on the same (rounded) operands, and bit for bit against the Linear over a gathered copy of the
+    blocks that it replaces (pvt_dge.py:62, :81-83, :164, :175)."""
+    from vtpack_amd import engine, ops
+    g = torch.Generator().manual_seed(H * W + C + k)
+    x = torch.randn((B, H * W, C), generator=g).to(dtype)
+    w4 = (torch.randn((N, C, k, k), generator=g) / (k * C ** 0.5)).to(dtype)
+    b = torch.randn((N,), generator=g).to(dtype)
+    wk = w4.permute(0, 2, 3, 1).reshape(N, -1).contiguous()
+    xd, wd, bd = x.to(dev), wk.to(dev), b.to(dev)
+    assert ops.fits_patch_linear(xd, H, W, k, wd, bd)
+    got = ops.patch_linear(xd, H, W, k, wd, bd)
+    want = F.conv2d(x.double().view(B, H, W, C).permute(0, 3, 1, 2), w4.double(), b.double(), stride=k)
+    want = want.permute(0, 2, 3, 1).reshape(-1, N)
+    assert_close(got, want, dtype, "patch_linear")
+    old = ops.linear(engine.tokens_to_patches(xd, H, W, k), wd, bd)
+    assert torch.equal(got, old)
+
+
+def test_patch_linear_refusals(dev):
+    from vtpack_amd import ops
+    x = torch.zeros((2, 64, 48), device=dev, dtype=torch.bfloat16)      # 96-byte token rows: no whole 128-byte pieces
+    w = torch.zeros((64, 4 * 48), device=dev, dtype=torch.bfloat16)
+    b = torch.zeros((64,), device=dev, dtype=torch.bfloat16)
+    assert not ops.fits_patch_linear(x, 8, 8, 2, w, b)
+    with pytest.raises(ValueError):
+        ops.patch_linear(x, 8, 8, 2, w, b)
+    x = torch.zeros((2, 64, 64), device=dev, dtype=torch.bfloat16)
+    w = torch.zeros((64, 9 * 64), device=dev, dtype=torch.bfloat16)
+    assert not ops.fits_patch_linear(x, 8, 8, 3, w, b)                   # the grid is not a multiple of the block
+    assert not ops.fits_patch_linear(x, 8, 8, 2, w, None)

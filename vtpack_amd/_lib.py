@@ -37,6 +37,7 @@ SIGNATURES = {
     "vtdge_layernorm": [_p, _p, _p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_linear": [_p, _l, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],
     "vtdge_patch_embed": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p],
+    "vtdge_patch_linear": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_linear_packed_size": [_i, _i, _i, _p],
     "vtdge_linear_prepack": [_p, _i, _i, _i, _p, _p],
     "vtdge_linear_prepacked": [_p, _l, _p, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],

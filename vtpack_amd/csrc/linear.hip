@@ -192,6 +192,13 @@ template <typename T>
 int launch_patch_embed(const void *images, const void *W, const void *bias, const void *pos, void *out, int B, int Cin,
                        int S, int P, int N, int extra, hipStream_t st);
 
+// a strided convolution over a channels-last token grid on the same kernel (linear_dma.hip)
+bool patch_linear_applicable(int P, int H, int W, int C, int N, int esz, const void *tokens, const void *weight,
+                             const void *bias, const void *out);
+template <typename T>
+int launch_patch_linear(const void *tokens, const void *W, const void *bias, void *out, int B, int H, int Wd, int C,
+                        int P, int N, hipStream_t st);
+
 // weight-stationary variant for bf16, K = 384 (linear_ws8.hip)
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out);
@@ -415,4 +422,21 @@ extern "C" int vtdge_patch_embed(const void *images, const void *weight, const v
     if (dtype == VTDGE_F32)
         return launch_patch_embed<float>(images, weight, bias, pos_embed, tokens, B, Cin, S, P, C, extra, st);
     return launch_patch_embed<bf16_t>(images, weight, bias, pos_embed, tokens, B, Cin, S, P, C, extra, st);
+}
+
+extern "C" int vtdge_patch_linear(const void *tokens, const void *weight, const void *bias, void *out, int B, int H,
+                                  int W, int C, int P, int N, int dtype, void *stream)
+{
+    VT_REQUIRE(tokens && weight && out, VTDGE_ERR_ARG, "patch_linear: NULL operand");
+    VT_REQUIRE(dtype == VTDGE_F32 || dtype == VTDGE_BF16, VTDGE_ERR_ARG, "patch_linear: unknown dtype %d", dtype);
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && C > 0 && P > 0 && N > 0, VTDGE_ERR_ARG, "patch_linear: bad sizes");
+    const int esz = dtype == VTDGE_F32 ? 4 : 2;
+    VT_REQUIRE(patch_linear_applicable(P, H, W, C, N, esz, tokens, weight, bias, out), VTDGE_ERR_UNSUPPORTED,
+               "patch_linear: no kernel for a %d x %d block of a %d x %d grid of %d channels, width %d (or bias missing, "
+               "or an operand not 16-byte aligned)", P, P, H, W, C, N);
+    VT_REQUIRE((int64_t)B * H * W < (1ll << 31) && (int64_t)B * H * W * C < (1ll << 40), VTDGE_ERR_UNSUPPORTED,
+               "patch_linear: batch too large");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VTDGE_F32) return launch_patch_linear<float>(tokens, weight, bias, out, B, H, W, C, P, N, st);
+    return launch_patch_linear<bf16_t>(tokens, weight, bias, out, B, H, W, C, P, N, st);
 }

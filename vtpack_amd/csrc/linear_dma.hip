@@ -69,8 +69,15 @@ template <> __device__ __forceinline__ float gelu_fn<bf16_t>(float v)
 // their per-lane source addresses differs from the plain kernel, no unfolded copy of the images exists.  The output
 // row goes to token `extra + gy G + gx` of sample b in [B, extra + G G, N], and the residual is row
 // `extra + gy G + gx` of one [extra + G G, N] table for every sample (the position embedding).
+//
+// The same mode reads patches of a channels-last token grid (cl_C > 0): A is [B, cl_H cl_W, cl_C] tokens, row
+// (b, gy, gx) of the product is the P x P block of tokens at (gy P, gx P) and its K index runs over (token row of
+// the block, token of that row, channel), i.e. a 128-byte K slab is a piece of one token's channels (cl_C values
+// must fill whole slabs).  This is a stride-P P x P convolution over the grid with its weight in [O, kh, kw, C]
+// order; rows of the product are stored densely (extra = 0) and there is no residual.
 struct PatchGeom {
     int P, S, G, Cin, extra;     // patch edge, image edge, patches per edge, input channels, tokens in front
+    int cl_C, cl_H, cl_W;        // channels-last source: channels and token grid (cl_C = 0: an image batch)
 };
 
 template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HAS_BIAS, bool HAS_RES, int NSTAGE = 3,
@@ -123,12 +130,21 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
                     int64_t gm = m0 + r;
                     gm = gm < M ? gm : M - 1;
                     if constexpr (PATCH) {
-                        // patch (b, gy, gx); the chunk is pixels `cc` of patch row `cr` of the slab's first rows
-                        const int g2 = pg.G * pg.G, cpr = pg.P * ESZ / 16;      // chunks per patch row
-                        const int gmi = (int)gm, b = gmi / g2, t = gmi - b * g2, gy = t / pg.G, gx = t - gy * pg.G;
-                        const int cr = chunk / cpr, cc = chunk % cpr;
-                        src[i] = reinterpret_cast<const unsigned char *>(
-                                     A + ((int64_t)b * pg.Cin * pg.S + gy * pg.P + cr) * pg.S + gx * pg.P) + cc * 16;
+                        if (pg.cl_C > 0) {
+                            // block (b, gy, gx) of the token grid: its first token; the slab's piece is added per stage
+                            const int gw = pg.cl_W / pg.P, g2 = (pg.cl_H / pg.P) * gw;
+                            const int gmi = (int)gm, b = gmi / g2, t = gmi - b * g2, gy = t / gw, gx = t - gy * gw;
+                            src[i] = reinterpret_cast<const unsigned char *>(
+                                         A + (((int64_t)b * pg.cl_H + gy * pg.P) * pg.cl_W + gx * pg.P) * pg.cl_C) +
+                                     chunk * 16;
+                        } else {
+                            // patch (b, gy, gx); the chunk is pixels `cc` of patch row `cr` of the slab's first rows
+                            const int g2 = pg.G * pg.G, cpr = pg.P * ESZ / 16;      // chunks per patch row
+                            const int gmi = (int)gm, b = gmi / g2, t = gmi - b * g2, gy = t / pg.G, gx = t - gy * pg.G;
+                            const int cr = chunk / cpr, cc = chunk % cpr;
+                            src[i] = reinterpret_cast<const unsigned char *>(
+                                         A + ((int64_t)b * pg.Cin * pg.S + gy * pg.P + cr) * pg.S + gx * pg.P) + cc * 16;
+                        }
                     } else {
                         src[i] = reinterpret_cast<const unsigned char *>(A + gm * lda) + chunk * 16;
                     }
@@ -145,9 +161,16 @@ __global__ __launch_bounds__((WGM * WGN + NWP) * 64) void linear_dma_kernel(
             unsigned char *dst = smem + (issued % NSTAGE) * STAGE + lw * NLW * 1024;
             int64_t a_off = (int64_t)it_kt * DKB;
             if constexpr (PATCH) {
-                // slab it_kt of a patch: its channel and its first row in the patch
-                const int rps = DKB / (pg.P * ESZ), spc = pg.P / rps;          // rows per slab, slabs per channel
-                a_off = ((int64_t)(it_kt / spc) * pg.S + (it_kt % spc) * rps) * pg.S * ESZ;
+                if (pg.cl_C > 0) {
+                    // slab it_kt of a block of tokens: which token of the block and where in its channels
+                    const int spt = pg.cl_C * ESZ / DKB;                       // slabs per token
+                    const int tk = it_kt / spt, dy = tk / pg.P, dx = tk - dy * pg.P;
+                    a_off = ((int64_t)(dy * pg.cl_W + dx) * pg.cl_C) * ESZ + (int64_t)(it_kt - tk * spt) * DKB;
+                } else {
+                    // slab it_kt of a patch: its channel and its first row in the patch
+                    const int rps = DKB / (pg.P * ESZ), spc = pg.P / rps;      // rows per slab, slabs per channel
+                    a_off = ((int64_t)(it_kt / spc) * pg.S + (it_kt % spc) * rps) * pg.S * ESZ;
+                }
             }
 #pragma unroll
             for (int i = 0; i < NLW; i++) {
@@ -319,7 +342,7 @@ struct LinArgs {
 };
 
 template <typename T, int BM, int BN, int WGM, int WGN, int NWP, int ACT, bool HB, bool HR, bool PATCH = false>
-static int go(const LinArgs &a, const PatchGeom &pg = PatchGeom{0, 0, 0, 0, 0})
+static int go(const LinArgs &a, const PatchGeom &pg = PatchGeom{0, 0, 0, 0, 0, 0, 0, 0})
 {
     constexpr int NW = WGM * WGN + NWP;
     constexpr int NSTAGE = (size_t)3 * (BM + BN) * DKB <= 160 * 1024 ? 3 : 2;
@@ -391,7 +414,7 @@ int launch_patch_embed(const void *images, const void *W, const void *bias, cons
                        int S, int P, int N, int extra, hipStream_t st)
 {
     const int G = S / P;
-    const PatchGeom pg{P, S, G, Cin, extra};
+    const PatchGeom pg{P, S, G, Cin, extra, 0, 0, 0};
     LinArgs a{images, 0, W, bias, pos, N, out, N, nullptr, (int64_t)B * G * G, N, Cin * P * P, VTDGE_ACT_NONE, st};
     // 256x128 tiles (half the passes over the weights, one workgroup per CU) once they give every CU two tiles and
     // more; 128x128 tiles, two workgroups per CU, for smaller batches.  At 256 x 256 patches and N = 384: 67 against
@@ -400,6 +423,33 @@ int launch_patch_embed(const void *images, const void *W, const void *bias, cons
         return go<T, 256, 128, 4, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
     return go<T, 128, 128, 2, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
 }
+
+// A stride-P P x P convolution over a channels-last token grid [B, H W, C] (weight in [N, kh, kw, C] order) + bias:
+// rows (b, gy, gx) of out [B (H/P) (W/P), N].
+bool patch_linear_applicable(int P, int H, int W, int C, int N, int esz, const void *tokens, const void *weight,
+                             const void *bias, const void *out)
+{
+    return P > 0 && H > 0 && W > 0 && H % P == 0 && W % P == 0 && ((int64_t)C * esz) % DKB == 0 &&
+           N % (16 / esz) == 0 && bias != nullptr &&
+           (((uintptr_t)tokens | (uintptr_t)weight | (uintptr_t)bias | (uintptr_t)out) & 15) == 0;
+}
+
+template <typename T>
+int launch_patch_linear(const void *tokens, const void *W, const void *bias, void *out, int B, int H, int Wd, int C,
+                        int P, int N, hipStream_t st)
+{
+    const PatchGeom pg{P, 0, 1, 0, 0, C, H, Wd};
+    const int64_t rows = (int64_t)B * (H / P) * (Wd / P);
+    LinArgs a{tokens, 0, W, bias, nullptr, 0, out, N, nullptr, rows, N, P * P * C, VTDGE_ACT_NONE, st};
+    if (N >= 768 || ceil_div(rows, 256) * ceil_div(N, 128) >= 512)
+        return go<T, 256, 128, 4, 2, 4, VTDGE_ACT_NONE, true, false, true>(a, pg);
+    return go<T, 128, 128, 2, 2, 4, VTDGE_ACT_NONE, true, false, true>(a, pg);
+}
+
+template int launch_patch_linear<float>(const void *, const void *, const void *, void *, int, int, int, int, int, int,
+                                        hipStream_t);
+template int launch_patch_linear<bf16_t>(const void *, const void *, const void *, void *, int, int, int, int, int, int,
+                                         hipStream_t);
 
 template int launch_patch_embed<float>(const void *, const void *, const void *, const void *, void *, int, int, int,
                                        int, int, int, hipStream_t);

@@ -92,6 +92,15 @@ def tokens_to_patches(x, H, W, k):
     return x.reshape(B, H // k, k, W // k, k, C).permute(0, 1, 3, 2, 4, 5).reshape(B * (H // k) * (W // k), k * k * C)
 
 
+def _strided_conv(x, H, W, k, conv):
+    """Conv2d(k, stride k) over the channels-last token grid x [B, H*W, C] -> [B*(H/k)*(W/k), O], as a Linear over
+    the k x k blocks of tokens: read in place where the kernel takes the shape, else from a gathered copy."""
+    w = _khwc_weight(conv)
+    if FUSE_PATCH_EMBED and ops.fits_patch_linear(x, H, W, k, w, conv.bias):
+        return ops.patch_linear(x, H, W, k, w, conv.bias)
+    return ops.linear(tokens_to_patches(x, H, W, k), w, conv.bias)
+
+
 def _key_value_source(attn, x_ln, H, W, extra):
     """Tokens the keys and values are projected from: LN1(x) itself, or, with spatial reduction
     (vtpack/models/dge/pvt_dge.py:83-87), LayerNorm(Conv2d(C, C, sr, stride sr)(LN1(x))) with the convolution run
@@ -104,7 +113,7 @@ def _key_value_source(attn, x_ln, H, W, extra):
     if H % sr or W % sr:
         raise ValueError(f"token grid {H}x{W} is not a multiple of the reduction ratio {sr}")
     B, _, C = x_ln.shape
-    red = ops.linear(tokens_to_patches(x_ln, H, W, sr), _khwc_weight(attn.sr), attn.sr.bias)
+    red = _strided_conv(x_ln, H, W, sr, attn.sr)
     return ops.layernorm(red, attn.norm.weight, attn.norm.bias, attn.norm.eps).view(B, -1, C)
 
 
@@ -318,7 +327,7 @@ def pvt_forward(model, images):
         else:
             if H % k or W % k:
                 raise ValueError(f"token grid {H}x{W} is not a multiple of the stage's patch size {k}")
-            tok = ops.linear(tokens_to_patches(x, H, W, k), _khwc_weight(pe.proj), pe.proj.bias)
+            tok = _strided_conv(x, H, W, k, pe.proj)
             H, W = H // k, W // k
         C = tok.shape[-1]
         tok = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps).view(B, H * W, C)

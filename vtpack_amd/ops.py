@@ -450,6 +450,40 @@ def patch_embed(images, weight, bias, pos_embed, patch, extra, out=None):
     return out
 
 
+def fits_patch_linear(x, H, W, k, weight, bias):
+    """Whether `patch_linear` has a kernel: contiguous tokens whose channels fill whole 128-byte pieces, a grid that
+    is a multiple of the block edge, a bias."""
+    if x.dim() != 3 or bias is None or x.dtype not in (torch.float32, torch.bfloat16):
+        return False
+    esz = x.element_size()
+    C = x.shape[-1]
+    return (k > 0 and H > 0 and W > 0 and x.shape[1] == H * W and H % k == 0 and W % k == 0 and (C * esz) % 128 == 0
+            and weight.dim() == 2 and weight.shape[1] == k * k * C and weight.shape[0] % (16 // esz) == 0)
+
+
+def patch_linear(x, H, W, k, weight, bias, out=None):
+    """[B * (H/k) * (W/k), N]: the stride-k k x k convolution over the channels-last token grid x [B, H*W, C], as a
+    Linear over its k x k blocks of tokens read in place; `weight` [N, k*k*C] is the convolution's weight in
+    (kh, kw, c) order.  Replaces the spatial-reduction Conv2d and the later stages' PatchEmbed Conv2d
+    (vtpack/models/dge/pvt_dge.py:62, :81-83, :164, :175) without a gathered copy of the tokens."""
+    _need_gpu(x, weight, bias)
+    _check_like(x, weight=weight, bias=bias, out=out)
+    if not fits_patch_linear(x, H, W, k, weight, bias):
+        raise ValueError("patch_linear: no kernel for these operands (see fits_patch_linear)")
+    B, _, C = x.shape
+    N = weight.shape[0]
+    _check_vector("bias", bias, N)
+    x = _contig(x)
+    rows = B * (H // k) * (W // k)
+    if out is None:
+        out = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != (rows, N) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous tensor of shape {(rows, N)}")
+    call("vtdge_patch_linear", ptr(x), ptr(_contig(weight)), ptr(_contig(bias)), ptr(out), B, H, W, C, k, N,
+         dtype_code(x), stream_ptr(), tag=("patch_linear", B, H, W, C, k, N))
+    return out
+
+
 def linear_layernorm(a, records, weight, bias, ln_weight, ln_bias, act="none", rows_dev=None, out=None):
     """out = act(LayerNorm(a) @ weight.T + bias) from the raw rows a [..., 384] and their statistics records (from
     `layernorm_stats` or from the kernel that produced the rows): no normalised copy of `a` is written or read.
