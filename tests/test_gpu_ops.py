@@ -31,10 +31,12 @@ def _t(a, dev, dtype=None):
     (33, 4, 4, 1, [2, 1]),
     (7, 4, 4, 1, [1]),
     (2, 20, 20, 1, [4, 2, 1]),    # > 256 regions per sample: several passes of the LDS scan
-    (1500, 4, 4, 1, [4, 2, 1]),   # > 1024 samples: several passes of the sample scan (two-kernel path)
+    (1500, 4, 4, 1, [4, 2, 1]),   # count kernel + a write kernel that sums the lengths before its sample
+    (256, 14, 14, 0, [4, 2, 1]),  # PVT stage 1 at batch 256: 50176 regions, the same two kernels
+    (4097, 2, 2, 1, [4, 2, 1]),   # > 4096 samples: the one-workgroup count-and-scan in several passes, then the write
     (256, 4, 4, 1, [4, 2, 1]),    # the headline batch: one launch, every sample sums the counts before it
     (64, 8, 8, 1, [4, 2, 1]),
-    (300, 8, 8, 0, [4, 2, 1]),    # 19200 regions: just past the single-launch limit
+    (300, 8, 8, 0, [4, 2, 1]),    # 19200 regions: just past the single-launch limit (count kernel + write)
 ])
 def test_index_to_patch_bit_exact(dev, B, Hr, Wr, extra, splits):
     from vtpack_amd import _C

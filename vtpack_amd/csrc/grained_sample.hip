@@ -283,6 +283,33 @@ __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *_
     if (threadIdx.x == 0) offsets[B] = carry_s;
 }
 
+// Step 1 for batches of a few thousand samples: a wave per sample adds up the query counts of its regions ->
+// lengths; the write kernel then finds each sample's first row from the lengths before it (no scan, and no single
+// workgroup that reads every gate index of the batch).
+__global__ __launch_bounds__(256) void patch_count_kernel(const int64_t *__restrict__ indices,
+                                                           const int64_t *__restrict__ splits, int B, int nreg, int S,
+                                                           int extra, int64_t *__restrict__ lengths)
+{
+    __shared__ int sq[VTDGE_MAX_SPLITS];
+    if (threadIdx.x < VTDGE_MAX_SPLITS) {
+        const int ps = threadIdx.x < S ? (int)splits[threadIdx.x] : 0;
+        sq[threadIdx.x] = ps * ps;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= B) return;
+    int part = 0;
+    for (int i = lane; i < nreg; i += WAVE) {
+        int64_t g = indices[(int64_t)b * nreg + i];
+        g = g < 0 ? 0 : (g >= S ? S - 1 : g);
+        part += sq[g];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, WAVE);
+    if (lane == 0) lengths[b] = (int64_t)part + extra;
+}
+
 // Step 2: one workgroup per sample.  The per-region query counts go through an
 // LDS-staged wavefront prefix sum (256 regions per pass); then every thread emits
 // one descriptor per turn (row j of the sample: its region by binary search in the
@@ -291,6 +318,9 @@ __global__ __launch_bounds__(1024) void patch_count_scan_kernel(const int64_t *_
 // FUSED: the workgroup also finds its own first row, as the sum of the query counts of all samples before it (it
 // reads their gate indices itself: a few KB out of L2 for the batch sizes this variant is launched for), and writes
 // offsets / lengths; no first step then, and no dependency between workgroups.
+// Not FUSED: the first row comes from `offsets` (written by the scan kernel) or, with from_lengths, is the sum of
+// the lengths of the samples before this one (written by the count kernel), in which case the workgroup writes
+// offsets as well.
 typedef long long i64x2 __attribute__((ext_vector_type(2)));
 
 template <bool FUSED>
@@ -298,7 +328,8 @@ __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restr
                                                            const int64_t *__restrict__ splits,
                                                            int64_t *__restrict__ offsets, int64_t *__restrict__ lengths,
                                                            int Hr, int Wr, int S, int R, int extra,
-                                                           int64_t *__restrict__ patches, int64_t capacity)
+                                                           int64_t *__restrict__ patches, int64_t capacity,
+                                                           int from_lengths)
 {
     __shared__ int wave_tot[4];
     __shared__ int carry_s;
@@ -349,6 +380,18 @@ __global__ __launch_bounds__(256) void patch_write_kernel(const int64_t *__restr
         __syncthreads();
         row0 = before_s[0] + before_s[1] + before_s[2] + before_s[3] + (int64_t)b * extra;
         if (threadIdx.x == 0) offsets[b] = row0;
+    } else if (from_lengths) {
+        int64_t part = 0;
+        for (int i = threadIdx.x; i < b; i += 256) part += lengths[i];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, WAVE);
+        if (lane == 0) before_s[wid] = part;
+        __syncthreads();
+        row0 = before_s[0] + before_s[1] + before_s[2] + before_s[3];
+        if (threadIdx.x == 0) {
+            offsets[b] = row0;
+            if (b == (int)gridDim.x - 1) offsets[b + 1] = row0 + lengths[b];
+        }
     } else {
         row0 = offsets[b];
     }
@@ -1265,14 +1308,22 @@ extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *split
     if (patches != nullptr && (int64_t)B * Hr * Wr <= 16384) {
         // small batches: one launch, every sample's workgroup sums the counts before it on its own
         patch_write_kernel<true><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
-                                                    capacity_rows);
+                                                    capacity_rows, 0);
         return check_launch("index_to_patch");
+    }
+    if (patches != nullptr && B <= 4096) {
+        // a wave per sample counts, then every sample's workgroup sums the lengths before it (a few KB)
+        patch_count_kernel<<<(B + 3) / 4, 256, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, lengths);
+        if (int rc = check_launch("index_to_patch(count)")) return rc;
+        patch_write_kernel<false><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
+                                                     capacity_rows, 1);
+        return check_launch("index_to_patch(write)");
     }
     patch_count_scan_kernel<<<1, 1024, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, offsets, lengths);
     if (int rc = check_launch("index_to_patch(count+scan)")) return rc;
     if (patches != nullptr) {
         patch_write_kernel<false><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
-                                                     capacity_rows);
+                                                     capacity_rows, 0);
         return check_launch("index_to_patch(write)");
     }
     return VTDGE_OK;
