@@ -875,12 +875,13 @@ __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T
         if (act) {
 #pragma unroll
             for (int j = 0; j < NJ; j++) {
-                ir[j] = *reinterpret_cast<const u32x4 *>(in + (r0 + j0 + j) * (int64_t)C);
-                if constexpr (SUB) sr[j] = *reinterpret_cast<const u32x4 *>(sub + (r0 + j0 + j) * (int64_t)C);
+                ir[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(in + (r0 + j0 + j) * (int64_t)C));
+                if constexpr (SUB)
+                    sr[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(sub + (r0 + j0 + j) * (int64_t)C));
             }
 #pragma unroll
             for (int dx = 0; dx < 4; dx++)
-                xr[dx] = *reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C);
+                xr[dx] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C));
         }
         // in - sub, rounded to the storage type (kept packed: four registers per row)
         if constexpr (SUB) {
