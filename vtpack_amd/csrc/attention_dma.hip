@@ -432,7 +432,7 @@ __global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_ke
                 const int chunk = lchunk ^ (is_v ? 2 * (r & 3) : (r >> 1) & 7);
                 off = (uint32_t)((r < n ? r : n - 1) * row_bytes + chunk * 16);
             }
-            dma16(is_v ? vbase : kbase, off, lds + j * 1024);
+            dma16_nt(is_v ? vbase : kbase, off, lds + j * 1024);
         }
     };
 

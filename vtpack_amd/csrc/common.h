@@ -193,6 +193,12 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t l
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base)
                  : "memory", "m0");
 }
+// the same for data that is read once and not again (streamed past the caches' reuse-oriented replacement)
+__device__ __forceinline__ void dma16_nt(const void *base, uint32_t off, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(off), "s"(base)
+                 : "memory", "m0");
+}
 // a wave-uniform pointer as the scalar register pair an address operand of the direct loads needs
 __device__ __forceinline__ const void *uniform_ptr(const void *p)
 {
