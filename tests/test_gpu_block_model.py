@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import torch_ref
-from util import FP32_REL, abs_err, assert_close, randn, rel_err
+from util import FP32_REL, LaunchNames, abs_err, assert_close, forced_reference, randn, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -107,16 +107,7 @@ def _gate_report(model, traces):
     return same, total, worst_margin
 
 
-def _forced_reference(model, images, heads, depth):
-    """Run the CPU path with the GPU's gate choices forced; every layer's trace also carries the logits the CPU
-    path's own router computes on its own activations (`gate_free`)."""
-    sd = torch_ref.float_state_dict(model)
-    forced = [blk.dge.states["gate"].float().argmax(-1).cpu() for blk in model.blocks]
-    traces = []
-    logits = torch_ref.deit_dge_forward(sd, images, heads, depth, forced_indices=forced, traces=traces)
-    for tr in traces:
-        tr["gate_free"] = tr["gate"]
-    return logits, traces
+_forced_reference = forced_reference
 
 
 def _assert_bf16_gates_differ_only_at_near_ties(model, traces, floor):
@@ -234,6 +225,31 @@ def test_deit_small_bf16_model(dev):
     want, traces = _forced_reference(m, img.float(), 6, 12)
     _assert_bf16_gates_differ_only_at_near_ties(m, traces, 0.97)
     assert_close(got.float(), want, torch.bfloat16, "DeiT-S+DGE bf16 logits")
+
+
+def test_deit_small_bf16_model_on_the_weight_stationary_kernels(dev):
+    """The same comparison at batch 8: 2056 token rows, the smallest batch at which the 256 px model takes the path
+    the headline measurement runs - both LayerNorms folded into weight-stationary Linears, proj writing the
+    statistics records, the scatter-back routing the next block and writing the records of its tokens, attention with
+    resident keys and values - instead of the streaming Linear and standalone LayerNorms of smaller batches."""
+    from vtpack_amd import _lib
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_small_patch16_256", dev, torch.bfloat16, seed=4)
+    img = synthetic_images(8, 256, seed=5, dtype=torch.bfloat16)
+    _lib.timer = names = LaunchNames()
+    try:
+        with torch.no_grad():
+            got = m(img.to(dev))
+    finally:
+        _lib.timer = None
+    assert names.names.count("vtdge_linear_layernorm") == 24 and names.names.count("vtdge_linear_stats") == 12
+    assert names.names.count("vtdge_decompress_router") == 11 and names.names.count("vtdge_layernorm") == 1
+    want, traces = forced_reference(m, img.float(), 6, 12)
+    for blk, tr in zip(m.blocks, traces):
+        assert torch.equal(blk.dge.states["patches"].cpu(), tr["patches"])
+        assert torch.equal(blk.dge.states["batches"], tr["lengths"])
+    _assert_bf16_gates_differ_only_at_near_ties(m, traces, 0.97)
+    assert_close(got.float(), want, torch.bfloat16, "DeiT-S+DGE bf16 logits, batch 8")
 
 
 def test_high_res_geometry(dev):

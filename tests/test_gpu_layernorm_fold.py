@@ -216,7 +216,9 @@ def test_linear_writes_records_of_its_rows(dev, live, has_bias, has_res):
     g = torch.Generator().manual_seed(7 + (live or 0))
     a = torch.randn(M, C, generator=g).bfloat16().to(dev)
     w = (torch.randn(C, C, generator=g) * 0.05).bfloat16().to(dev)
-    b = (torch.randn(C, generator=g) * 0.2).bfloat16().to(dev) if has_bias else None
+    # a bias far from zero: without a residual it is what moves the rows' means away from zero (|mean| ~ 30 sigma), the
+    # case the pivoted sums are there for
+    b = (torch.randn(C, generator=g) * 0.2 + (0.0 if has_res else 30.0)).bfloat16().to(dev) if has_bias else None
     res = (torch.randn(M, C, generator=g) * 2 + 3 * torch.randn(M, 1, generator=g)).bfloat16().to(dev) if has_res else None
     rows_dev = None if live is None else torch.tensor([live], dtype=torch.int64, device=dev)
     L = M if live is None else live
@@ -233,7 +235,7 @@ def test_linear_writes_records_of_its_rows(dev, live, has_bias, has_res):
     mean, sigma, _ = decode(rec[:L])
     m_ref, s_ref = want_stats(want)
     assert_record_layout(rec[:L])
-    assert float((mean.double() - m_ref).abs().max()) < 1e-5
+    assert float((mean.double() - m_ref).abs().max()) < 1e-5 * max(1.0, float(m_ref.abs().max()) / 8)
     assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
 
 
@@ -302,21 +304,13 @@ def test_scatter_records_refused_for_other_rows(dev):
 def test_model_with_and_without_folded_norms(dev):
     """DeiT-S+DGE, bf16, 256 px, batch 16 (enough rows for the weight-stationary kernels): with the folding on the
     forward launches one statistics kernel (the first block's tokens) and one LayerNorm (the final one) instead of 25
-    LayerNorms; the routing of the first block is the same either way and, while the routing stays the same, the
-    logits agree within the bf16 bar."""
+    LayerNorms.  Rounding differs between the two forms, so a near-tie of some router may fall the other way and the
+    two runs need not route alike after the first block: each run is therefore compared with the CPU restatement
+    under its OWN gate choices (logits within the bf16 bar, integer outputs of every layer exact)."""
     from vtpack_amd import _lib, engine
     from vtpack_amd.models import dge as zoo
     from vtpack_amd.synthetic import set_synthetic_router, synthetic_images
-
-    class Count:
-        def __init__(self):
-            self.names = []
-
-        def begin(self, name, tag):
-            self.names.append(name)
-
-        def end(self):
-            pass
+    from util import LaunchNames, forced_reference
 
     torch.manual_seed(0)
     m = zoo.deit_dge_s124_small_patch16_256()
@@ -327,10 +321,17 @@ def test_model_with_and_without_folded_norms(dev):
     try:
         for fold in (True, False):
             engine.FOLD_NORMS = fold
-            _lib.timer = Count()
+            _lib.timer = LaunchNames()
             with torch.no_grad():
                 out = m(img)
-            runs[fold] = (out.float(), [blk.dge.states["batches_device"].clone() for blk in m.blocks], _lib.timer.names)
+            names = _lib.timer.names
+            _lib.timer = None
+            want, traces = forced_reference(m, img.float().cpu(), 6, 12)
+            for blk, tr in zip(m.blocks, traces):
+                assert torch.equal(blk.dge.states["patches"].cpu(), tr["patches"])
+                assert torch.equal(blk.dge.states["batches"], tr["lengths"])
+            assert abs_err(out.float(), want) <= BF16_ABS, f"folded LayerNorms {'on' if fold else 'off'}"
+            runs[fold] = (out.float(), [blk.dge.states["batches_device"].clone() for blk in m.blocks], names)
     finally:
         engine.FOLD_NORMS = True
         _lib.timer = None
@@ -338,7 +339,6 @@ def test_model_with_and_without_folded_norms(dev):
     assert names_off.count("vtdge_layernorm") == 25 and names_off.count("vtdge_linear_layernorm") == 0
     assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 1
     assert names_on.count("vtdge_linear_layernorm") == 24 and names_on.count("vtdge_linear_stats") == 12
-    assert bool(torch.isfinite(on).all())
     assert torch.equal(len_on[0], len_off[0])
     if all(torch.equal(a, b) for a, b in zip(len_on, len_off)):
         assert abs_err(on, off) <= 2 * BF16_ABS

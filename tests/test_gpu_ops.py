@@ -507,6 +507,47 @@ def test_sparse_attention(dev, dtype, B, h, d, n, lo, hi):
     assert_close(got.float(), want, dtype, "sparse attention")
 
 
+@pytest.mark.parametrize("n", [20, 32, 64, 96, 128, 160, 192, 196, 256, 257, 288])
+def test_sparse_attention_resident_keys_many_items(dev, n):
+    """bf16, head_dim 64, up to 288 keys: the kernel that keeps an item's keys and values in LDS, with more
+    (sample, head) items than compute units, so that every workgroup walks several items (double buffer, the next
+    item's keys / values and first query tile fetched under the current item's arithmetic, the item table in LDS).
+    One case per number of 32-key blocks (1 .. 9), with and without a partial last block; query counts mix empty
+    samples, single queries, counts around the 32-query tile and the 128-query half, and samples of more than 256
+    queries (a ninth tile, whose queries are loaded inside the loop)."""
+    from vtpack_amd import _C
+    B, h, d = 200, 3, 64
+    r = rng(700 + n)
+    lengths = r.choice([0, 1, 2, 31, 32, 33, 64, 100, 127, 128, 129, 200, 256, 257, 300], size=B,
+                       p=[.1, .1, .08, .08, .08, .08, .08, .08, .06, .06, .06, .05, .03, .03, .03]).astype(np.int64)
+    lengths[:4] = [300, 0, 257, 1]
+    L = int(lengths.sum())
+    q, k, v = bf16_round(randn(701, h, L, d)), bf16_round(randn(702, h, B, n, d)), bf16_round(randn(703, h, B, n, d))
+    scale = d ** -0.5
+    want = orc.attention(q, k, v, lengths, scale)
+    got = _C.batched_sparse_attention_forward(_t(q, dev, torch.bfloat16), _t(k, dev, torch.bfloat16),
+                                              _t(v, dev, torch.bfloat16), torch.from_numpy(lengths), scale)
+    assert got.shape == (h, L, d)
+    assert_close(got.float(), want, torch.bfloat16, f"sparse attention, {B * h} items of {n} keys")
+
+
+def test_sparse_attention_more_items_than_the_item_table_holds(dev):
+    """More than 512 items per workgroup (here 132 000 items of 8 keys): the first row and query count of an item
+    are then read from `offsets` inside the loop instead of from the table in LDS."""
+    from vtpack_amd import _C
+    B, h, d, n = 22000, 6, 64, 8
+    r = rng(710)
+    lengths = r.choice([0, 1, 2, 3, 40], size=B, p=[.3, .4, .2, .09, .01]).astype(np.int64)
+    L = int(lengths.sum())
+    fast = np.random.default_rng(711)             # 135 M values: the legacy generator would take 12 s over them
+    q, k, v = (bf16_round(fast.standard_normal(shape, dtype=np.float32)) for shape in ((h, L, d), (h, B, n, d), (h, B, n, d)))
+    scale = d ** -0.5
+    want = orc.attention(q, k, v, lengths, scale)
+    got = _C.batched_sparse_attention_forward(_t(q, dev, torch.bfloat16), _t(k, dev, torch.bfloat16),
+                                              _t(v, dev, torch.bfloat16), torch.from_numpy(lengths), scale)
+    assert_close(got.float(), want, torch.bfloat16, "sparse attention, 132 000 items")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_sparse_attention_strided_kv(dev, dtype):
     """q straight from the q Linear ([L, h*d]) and k, v as views of the kv Linear output ([B, n, 2, h, d])."""

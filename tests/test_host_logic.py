@@ -205,3 +205,44 @@ def test_budget_loss_from_planted_gates():
     assert float(ratio) == pytest.approx(1.0) and float(loss) == pytest.approx(0.0, abs=1e-12)
     # the per-encoder ratio of engine.py:20-32 on the same states
     assert float(harness.get_complexity(m)) == pytest.approx(1.0)
+
+
+def test_states_resolve_deferred_values_on_every_read_and_on_every_way_out():
+    """`states` hands out what the reference's plain dict would hold, however it is read, and a deferred value is
+    worked out again on every read (a graph replay rewrites the tensors behind it without running Python)."""
+    from vtpack_amd.layers.dge import Deferred, States
+    box = {"n": 3}
+    st = States({"plain": 7, "batches": Deferred(lambda: box["n"]), "comp": Deferred(lambda: list(range(box["n"])))})
+    assert st["batches"] == 3 and st.get("comp") == [0, 1, 2] and st.get("missing", 5) == 5
+    box["n"] = 2                                   # what a replay does: new counts, no Python
+    assert st["batches"] == 2 and st["comp"] == [0, 1]
+    assert isinstance(dict.__getitem__(st, "batches"), Deferred)       # nothing was stored back
+    for view in (dict(st), {**st}, st.copy(), st.snapshot(), dict(st.items()), dict(zip(st.keys(), st.values()))):
+        assert type(view) is dict and view == {"plain": 7, "batches": 2, "comp": [0, 1]}
+    snap = st.copy()
+    box["n"] = 4
+    assert snap["batches"] == 2 and st["batches"] == 4                 # a snapshot does not follow
+    assert st.setdefault("batches", 0) == 4 and st.setdefault("new", 9) == 9
+    assert st.pop("comp") == [0, 1, 2, 3] and "comp" not in st and st.pop("comp", None) is None
+    with pytest.raises(KeyError):
+        st.pop("comp")
+    seen = {}
+    while st:
+        k, v = st.popitem()
+        seen[k] = v
+    assert seen == {"plain": 7, "batches": 4, "new": 9}
+
+
+def test_fused_forward_refuses_a_distillation_token_without_a_class_token():
+    """The reference never builds that token order (deit_dge.py:270-275); layer mode raises in embed_tokens and the
+    fused forward must not run with the distillation token in the class token's place."""
+    from vtpack_amd import engine
+    from vtpack_amd.models.dge.deit_dge import VisionTransformer
+    m = VisionTransformer(img_size=32, patch_size=16, embed_dim=16, depth=1, num_heads=1, distilled=True,
+                          split_sizes=[2, 1]).eval()
+    m.cls_token = None
+    img = torch.zeros(1, 3, 32, 32)
+    with pytest.raises(ValueError, match="class token"):
+        engine.model_forward(m, img)
+    with pytest.raises(ValueError, match="class token"):
+        m.embed_tokens(img)

@@ -45,3 +45,30 @@ def randn(seed, *shape):
 def bf16_round(a):
     """fp32 numpy -> the fp32 value of its bf16 rounding (round to nearest even), via torch."""
     return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).float().numpy()
+
+
+def forced_reference(model, images, heads, depth):
+    """The CPU restatement of a DeiT+DGE forward with the GPU run's gate choices forced (read from the model's
+    `states` after its forward): -> (logits, per-layer traces).  Every layer's trace also carries the logits the CPU
+    path's own router computes on its own activations (`gate_free`)."""
+    from oracle import torch_ref
+    sd = torch_ref.float_state_dict(model)
+    forced = [blk.dge.states["gate"].float().argmax(-1).cpu() for blk in model.blocks]
+    traces = []
+    logits = torch_ref.deit_dge_forward(sd, images, heads, depth, forced_indices=forced, traces=traces)
+    for tr in traces:
+        tr["gate_free"] = tr["gate"]
+    return logits, traces
+
+
+class LaunchNames:
+    """A stand-in for the library's launch timer that only notes which entry points were called."""
+
+    def __init__(self):
+        self.names = []
+
+    def begin(self, name, tag):
+        self.names.append(name)
+
+    def end(self):
+        pass

@@ -31,8 +31,10 @@
 //   rstd = 1 / (sigma_1 + sigma_2).  A separate bias is not taken (it is part of b').
 //   HAS_STAT (one column group, N = 384: the workgroup owns whole output rows): also writes the statistics records
 //   of the output rows (fp32 values before their rounding to bf16), for a HAS_LN Linear that takes `out` next: sums
-//   about a pivot common to the row (the first element of its residual), added up over the four lanes of a row and,
-//   one barrier later, over the eight waves by a few lanes per wave, which write 128 contiguous bytes of records.
+//   about a pivot taken from the row itself (the first element of its residual; without a residual each wave's first
+//   output element of the row, the waves' sums being moved to one pivot when they are merged), added up over the four
+//   lanes of a row and, one barrier later, over the eight waves by a few lanes per wave, which write 128 contiguous
+//   bytes of records.
 //
 // Synchronisation: one s_barrier per tile.  Vector-memory operations retire in issue order; each wave keeps a tally
 // of the ones it has issued and, per tile, the tally right after that tile's direct loads, and waits with a counted
@@ -236,6 +238,12 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
         if constexpr (ACT == VTDGE_ACT_GELU) f = w8_gelu(f);
         if constexpr (HAS_STAT) {
             if (E == 0) sa = sq = 0.f;
+            if constexpr (!HAS_RES) {
+                // no residual to take the pivot from: the row's first output element of this wave's strip (lane
+                // kg = 0, E = 0), handed to the row's other lanes; the eight waves' pivots differ and are brought
+                // to a common one when their sums are merged
+                if (E == 0) pv[RB] = __shfl(f, c16, WAVE);
+            }
             const float dl = f - pv[RB];
             sa += dl;
             sq = fmaf(dl, dl, sq);
@@ -356,9 +364,18 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const u32x4 v = *reinterpret_cast<const u32x4 *>(pb + i * 512);
-            pivot = __uint_as_float(v.x);          // the same in all eight
-            sa += __uint_as_float(v.y);
-            sq += __uint_as_float(v.z);
+            if constexpr (HAS_RES) {
+                pivot = __uint_as_float(v.x);      // the same in all eight
+                sa += __uint_as_float(v.y);
+                sq += __uint_as_float(v.z);
+            } else {
+                // sums of 48 values about the wave's own pivot p_i, moved to wave 0's pivot P (d = p_i - P):
+                //   sum (x - P) = sa_i + 48 d,   sum (x - P)^2 = sq_i + 2 d sa_i + 48 d^2
+                if (i == 0) pivot = __uint_as_float(v.x);
+                const float d = __uint_as_float(v.x) - pivot, si = __uint_as_float(v.y);
+                sa += fmaf(48.0f, d, si);
+                sq += fmaf(d, fmaf(48.0f, d, 2.0f * si), __uint_as_float(v.z));
+            }
         }
         const float m = sa * (1.0f / 384.0f);
         const float var = fmaxf(sq * (1.0f / 384.0f) - m * m, 0.f);

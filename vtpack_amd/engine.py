@@ -1,7 +1,7 @@
 """Fused inference path of one DGE transformer block: every step on libvtdge kernels.
 
 What `Block.forward` of the reference does with ~30 library launches and one device->host copy
-(vtpack/models/dge/deit_dge.py:123-130) becomes 13 kernel launches on the caller's stream with the
+(vtpack/models/dge/deit_dge.py:123-130) becomes 9 kernel launches (on two streams, joined before attention) with the
 packed query count kept in device memory: buffers are sized for the worst case (one query per
 token) and every packed kernel reads the live row count itself.  Nothing here synchronises, so the
 whole forward can be captured into a HIP graph.
@@ -226,16 +226,13 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 
     # `states` as the reference's code reads it (vtpack/layers/dge.py:81-84): the host-side counts and the tensors cut
-    # to the live rows are produced on first read (one device->host copy, then cached); nothing is copied otherwise.
-    live = {}
-
+    # to the live rows are produced when they are read (one device->host copy per read, nothing cached: a graph replay
+    # rewrites `lengths` without running this code); nothing is copied otherwise.
     def batches():
-        if "n" not in live:
-            live["n"] = lengths.cpu()
-        return live["n"]
+        return lengths.cpu()
 
     def cut(t):
-        return lambda: t[:int(batches().sum())]
+        return lambda: t[:int(lengths.sum())]
 
     dge.states.update({"comp": Deferred(cut(comp)), "input": x, "patches": Deferred(cut(patches)),
                        "batches": Deferred(batches), "batches_device": lengths, "offsets_device": offsets,
@@ -272,6 +269,8 @@ def model_forward(model, images):
     G = S // P
     C = model.embed_dim
     front = [t for t in (model.cls_token, getattr(model, "dist_token", None)) if t is not None]
+    if model.cls_token is None and front:
+        raise ValueError("a distillation token needs a class token (deit_dge.py:270-275)")
     extra = len(front)
     if FUSE_PATCH_EMBED and ops.fits_patch_embed(images, pe.proj.weight, pe.proj.bias, model.pos_embed, P):
         # the convolution reads the images in place and adds the position embedding on its way out

@@ -32,26 +32,62 @@ class States(dict):
 
     The fused inference path never copies the query counts to the host and works on buffers sized for the worst
     case.  It therefore stores `batches` (CPU int64 lengths), `comp`, `patches` and `queries` as `Deferred` values:
-    reading one of them performs the device->host copy of the counts once and returns what the reference's code
-    expects, tensors cut to the live rows.  Code that never reads them never synchronises."""
+    reading one of them performs the device->host copy of the counts and returns what the reference's code expects,
+    tensors cut to the live rows.  Code that never reads them never synchronises.
 
-    def _resolve(self, key, value):
-        if isinstance(value, Deferred):
-            value = value.make()
-            dict.__setitem__(self, key, value)
-        return value
+    A Deferred value is worked out on EVERY read and never stored back: the tensors behind it are rewritten by
+    each replay of a captured HIP graph (which runs no Python), so a cached count would go stale.  Every way of
+    taking values out of the dict resolves them - indexing, get, items, values, pop, popitem, setdefault, copy,
+    dict(states), {**states} - so code written against the reference's plain dict never sees a Deferred object."""
+
+    @staticmethod
+    def _resolve(value):
+        return value.make() if isinstance(value, Deferred) else value
 
     def __getitem__(self, key):
-        return self._resolve(key, dict.__getitem__(self, key))
+        return self._resolve(dict.__getitem__(self, key))
 
     def get(self, key, default=None):
-        return self._resolve(key, dict.get(self, key, default)) if key in self else default
+        return self[key] if key in self else default
+
+    # overriding __iter__ / keys also takes dict(states) and {**states} off the C fast path, which would copy the
+    # raw values: they then go through keys() and __getitem__
+    def __iter__(self):
+        return dict.__iter__(self)
+
+    def keys(self):
+        return dict.keys(self)
 
     def items(self):
         return [(k, self[k]) for k in self.keys()]
 
     def values(self):
         return [self[k] for k in self.keys()]
+
+    def pop(self, key, *default):
+        if key in self:
+            value = self[key]
+            dict.__delitem__(self, key)
+            return value
+        if default:
+            return default[0]
+        raise KeyError(key)
+
+    def popitem(self):
+        key, value = dict.popitem(self)
+        return key, self._resolve(value)
+
+    def setdefault(self, key, default=None):
+        if key not in self:
+            dict.__setitem__(self, key, default)
+        return self[key]
+
+    def copy(self):
+        """A plain dict of the values as they are now (a snapshot: later forwards or graph replays do not change
+        it)."""
+        return {k: self[k] for k in self.keys()}
+
+    snapshot = copy
 
 
 class DynamicRouter(nn.Module):
