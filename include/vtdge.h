@@ -136,12 +136,36 @@ int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *p
  * split size must divide it; VTDGE_ERR_UNSUPPORTED for another R.
  * out_records (nullable) [B * (extra + H*W), 16] bf16: the statistics record of every row of `out` as stored (mean
  * and sqrt(var + records_eps), see vtdge_layernorm_stats), for the next block's norm1 -> kv through
- * vtdge_linear_layernorm; one-pass fp32 sums about a value of the row itself.  bf16 rows of 264 to 512 channels. */
+ * vtdge_linear_layernorm; one-pass fp32 sums about a value of the row itself.  bf16 rows of 264 to 512 channels.
+ * next_counts (nullable; needs the next router) uint8 [B * H/R * W/R]: the number of queries the next block takes
+ * from every region, next_splits[next_indices]^2 with next_splits int64 [S2] on the device: what
+ * vtdge_compress_regions adds up to place a region's queries. */
 int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits,
                             const int64_t *offsets, const void *ref, void *out, const void *next_weight,
                             const void *next_bias, void *next_gate, int64_t *next_indices, void *out_records,
-                            float records_eps, int B, int H, int W, int C, int extra, int R, int S, int S2, int dtype,
-                            void *stream);
+                            float records_eps, const int64_t *next_splits, uint8_t *next_counts, int B, int H, int W,
+                            int C, int extra, int R, int S, int S2, int dtype, void *stream);
+
+/* Gate indices -> packed queries in one step, by region: vtdge_index_to_patch and vtdge_compress together, i.e.
+ * grained_sample_index_to_patch followed by grained_sample_compress
+ * (vtpack/layers/csrc/grained_sample/grained_sample.cu:302-345 with :146-196, and :198-239 with :31-69) as
+ * DynamicGrainedEncoder.compress calls them (vtpack/layers/dge.py:76-79), without the descriptor list in between: a
+ * region's packed rows are consecutive, so the kernel places them from the query counts of the regions before it.
+ *   x [B, extra + H*W, C]   indices int64 [B, H/R, W/R]   splits int64 [S] (device)
+ *   counts  nullable uint8 [B * H/R * W/R, padded to a multiple of 16 bytes]: splits[indices]^2 per region, as
+ *           vtdge_decompress_router leaves them; without it the kernel works the counts out from `indices`
+ *   comp    [capacity_rows, C]: the packed queries, bit for bit those of vtdge_compress
+ *   records nullable [capacity_rows, 16] bf16: the statistics record of every row of comp as stored (mean and
+ *           sqrt(var + records_eps), see vtdge_layernorm_stats) for a vtdge_linear_layernorm that takes comp next
+ *           (norm1 -> q, vtpack/models/dge/deit_dge.py:127 with :72); bf16 only
+ *   patches (nullable), offsets [B+1], lengths [B]: as vtdge_index_to_patch writes them
+ * The caller guarantees capacity_rows >= the number of queries (B * (extra + H*W) always is).  R must be 4 with splits
+ * out of {1, 2, 4}, a row one 16-byte vector per lane (C <= 512 in bf16, 256 in fp32), at most 65536 regions and
+ * 64 extra tokens; VTDGE_ERR_UNSUPPORTED otherwise. */
+int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t *splits, const uint8_t *counts,
+                           void *comp, void *records, float records_eps, int64_t *patches, int64_t capacity_rows,
+                           int64_t *offsets, int64_t *lengths, int B, int H, int W, int C, int extra, int R, int S,
+                           int dtype, void *stream);
 
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */

@@ -336,9 +336,9 @@ def test_model_with_and_without_folded_norms(dev):
         engine.FOLD_NORMS = True
         _lib.timer = None
     (on, len_on, names_on), (off, len_off, names_off) = runs[True], runs[False]
-    assert names_off.count("vtdge_layernorm") == 25 and names_off.count("vtdge_linear_layernorm") == 0
+    assert names_off.count("vtdge_layernorm") == 37 and names_off.count("vtdge_linear_layernorm") == 0
     assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 1
-    assert names_on.count("vtdge_linear_layernorm") == 24 and names_on.count("vtdge_linear_stats") == 12
+    assert names_on.count("vtdge_linear_layernorm") == 36 and names_on.count("vtdge_linear_stats") == 12
     assert torch.equal(len_on[0], len_off[0])
     if all(torch.equal(a, b) for a, b in zip(len_on, len_off)):
         assert abs_err(on, off) <= 2 * BF16_ABS

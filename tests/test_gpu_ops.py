@@ -89,6 +89,90 @@ def test_compress_bit_exact(dev, dtype, B, H, W, extra, C):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("with_counts", [False, True])
+@pytest.mark.parametrize("B,H,W,extra,C,p", [(8, 16, 16, 1, 384, None), (2, 32, 32, 1, 384, None), (3, 8, 12, 0, 264, None),
+                                              (2, 16, 16, 2, 512, None), (300, 16, 16, 1, 384, [.6, .3, .1]),
+                                              (5, 4, 4, 1, 384, [0, 0, 1]), (4, 16, 16, 1, 384, [1, 0, 0]),
+                                              (64, 32, 32, 1, 384, [.2, .3, .5])])
+def test_compress_regions_bit_exact(dev, dtype, with_counts, B, H, W, extra, C, p):
+    """index->patch and compress as one kernel that works by region: the packed rows, descriptors, offsets and lengths
+    are those of the two operators (the oracle's), bit for bit, whether the rows before a region are added up from the
+    per-region count bytes or from the gate indices; the bytes themselves are checked where they come from (the
+    scatter-back that routes the next block)."""
+    from vtpack_amd import ops
+    if dtype == torch.float32:
+        C = C // 2                          # the same 16-byte vectors per row
+    idx = random_indices(B + C, B, H // 4, W // 4, p=p)
+    patches, lengths = orc.index_to_patch(idx, SPLITS, 4, extra)
+    x = randn(C + 1, B, extra + H * W, C)
+    x[0, 0, :8] = -0.0                      # 0 + (-0) = +0 in a window mean, -0 stays in a copied extra token
+    x[-1, -1, :8] = -0.0
+    if dtype == torch.bfloat16:
+        x = bf16_round(x)
+    want = torch.from_numpy(orc.compress(x, patches, H, W, extra)).to(dtype)
+    L = patches.shape[0]
+    counts = None
+    if with_counts:
+        counts = ops.region_counts_buffer(B, (H // 4) * (W // 4), dev)
+        counts.fill_(255)
+        counts[:idx.size] = torch.from_numpy((np.array(SPLITS)[idx.reshape(-1)] ** 2).astype(np.uint8)).to(dev)
+    sp = _t(np.array(SPLITS, dtype=np.int64), dev)
+    assert ops.fits_compress_regions(_t(x, dev, dtype), H, W, 4, SPLITS)
+    comp, rec, got_p, offsets, got_l = ops.compress_regions(_t(x, dev, dtype), _t(idx, dev), sp, H, W, 4, counts=counts)
+    assert rec is None and comp.dtype == dtype
+    assert torch.equal(got_l.cpu(), torch.from_numpy(lengths))
+    assert torch.equal(offsets.cpu(), torch.from_numpy(np.concatenate([[0], np.cumsum(lengths)])))
+    got_p, want_p = got_p[:L].cpu().numpy(), patches.copy()
+    ext = want_p[:, 1] < 0                  # column 2 of an extra token's row is unwritten in the reference: 0 here
+    assert np.array_equal(got_p[:, [0, 1, 3]], want_p[:, [0, 1, 3]]) and np.array_equal(got_p[~ext, 2], want_p[~ext, 2])
+    assert bool((got_p[ext, 2] == 0).all())
+    assert torch.equal(comp[:L].cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       want.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # and the two-kernel path of this library
+    p2, o2, l2 = ops.index_to_patch(_t(idx, dev), sp, 4, extra, capacity=B * (extra + H * W))
+    c2 = ops.compress(_t(x, dev, dtype), p2, W, extra, rows_dev=o2[B:], rows=B * (extra + H * W))
+    assert torch.equal(c2[:L], comp[:L]) and torch.equal(p2[:L], torch.from_numpy(got_p).to(dev))
+
+
+@pytest.mark.parametrize("B,H,W,extra,C", [(8, 16, 16, 1, 384), (2, 32, 32, 2, 512), (3, 8, 12, 0, 264)])
+def test_compress_regions_records(dev, B, H, W, extra, C):
+    """The statistics records of the packed rows as stored, for the q Linear with norm1 folded in."""
+    from vtpack_amd import ops
+    idx = random_indices(B, B, H // 4, W // 4)
+    g = torch.Generator().manual_seed(C)
+    x = (torch.randn(B, extra + H * W, C, generator=g) * 2 + 5 * torch.randn(B, extra + H * W, 1, generator=g))
+    x = x.bfloat16().to(dev)
+    sp = _t(np.array(SPLITS, dtype=np.int64), dev)
+    plain = ops.compress_regions(x, _t(idx, dev), sp, H, W, 4)
+    comp, rec, patches, offsets, lengths = ops.compress_regions(x, _t(idx, dev), sp, H, W, 4, stats_eps=1e-6)
+    L = int(offsets[-1])
+    assert torch.equal(comp[:L], plain[0][:L]) and torch.equal(patches[:L], plain[2][:L])
+    r = rec[:L].float()
+    mean, sigma = r[:, 0] + r[:, 2] + r[:, 5], r[:, 6] + r[:, 7]
+    cd = comp[:L].double()
+    m_ref, s_ref = cd.mean(1), (cd.var(1, unbiased=False) + 1e-6).sqrt()
+    assert bool((r[:, 0] == r[:, 1]).all() and (r[:, 0] == r[:, 3]).all() and (r[:, 2] == r[:, 4]).all())
+    assert bool((r[:, 6] == r[:, 8]).all() and (r[:, 7] == r[:, 9]).all() and (r[:, 10:] == 0).all())
+    assert float((mean.double() - m_ref).abs().max()) < 5e-6 * float(cd.abs().max())
+    assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
+
+
+def test_compress_regions_refuses_what_it_cannot_do(dev):
+    from vtpack_amd import ops
+    from vtpack_amd._lib import VtdgeError
+    x = torch.zeros(2, 65, 768, dtype=torch.bfloat16, device=dev)         # 96 vectors per row
+    idx = torch.zeros(2, 2, 2, dtype=torch.int64, device=dev)
+    sp = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    assert not ops.fits_compress_regions(x, 8, 8, 4, SPLITS)
+    assert not ops.fits_compress_regions(x[..., :384], 8, 8, 2, [2, 1])
+    assert not ops.fits_compress_regions(x[..., :64].contiguous(), 8, 8, 4, SPLITS)      # narrow rows: row-wise kernels
+    with pytest.raises(VtdgeError):
+        ops.compress_regions(x, idx, sp, 8, 8, 4)
+    with pytest.raises(TypeError):
+        ops.compress_regions(x[..., :384].float().contiguous(), idx, sp, 8, 8, 4, stats_eps=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("add_ref", [True, False])
 @pytest.mark.parametrize("B,H,W,extra,C", GEOMS)
 def test_decompress_bit_exact(dev, dtype, add_ref, B, H, W, extra, C):
@@ -667,6 +751,11 @@ def test_scatter_back_with_the_next_router(dev, dtype, B, Hr, Wr, C, extra):
                                                 next_bias=bias)
         assert torch.equal(got, want)
         assert torch.equal(nidx, want_idx) and torch.equal(gate, want_gate)
+    # the query counts of the next block's regions, a byte each, for compress_regions
+    got, gate, nidx, counts = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=None, next_weight=wgt,
+                                                    next_bias=bias, next_splits=splits)
+    assert torch.equal(nidx, want_idx) and counts.dtype == torch.uint8
+    assert torch.equal(counts[:nidx.numel()].long(), (splits[nidx.reshape(-1)] ** 2))
     # without a next router it is the plain scatter-back
     alone, g0, i0 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp)
     assert g0 is None and i0 is None

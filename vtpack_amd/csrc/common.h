@@ -314,6 +314,65 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// ---------------------------------------------------------------- statistics records of rows held by a wave
+// Lane exchanges of the record sums below: the value of the lane whose number differs in one bit.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// v summed over the lanes that differ in bits 2..5 of the lane number (16 of them), returned in each of them
+__device__ __forceinline__ float sum_over_lane_bits_2_to_5(float v)
+{
+    v += dpp_move<0x141>(dpp_move<0x1B>(v));      // lane ^ 4: the quad reversed, then the half row mirrored
+    v += dpp_move<0x128>(v);                      // lane ^ 8: the row rotated by eight
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);        // lane ^ 16: odd rows swapped with even rows
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);     // lane ^ 32: the halves swapped
+}
+// Statistics record of one stored row from the sums of (x - pivot) and (x - pivot)^2 over its C values, the pivot
+// being a value of the row itself (no cancellation however far the row's mean is from zero).
+__device__ __forceinline__ void row_record(float pivot, float s1, float s2, int C, float eps, u32x4 &lo, u32x4 &hi)
+{
+    const float m = s1 / (float)C;
+    const float var = fmaxf(s2 / (float)C - m * m, 0.f);
+    ln_record(pivot + m, sqrtf(var + eps), lo, hi);
+}
+// The records of FOUR rows that a wave holds side by side (every lane a piece of each row): st[2 t], st[2 t + 1] are
+// the lane's sums of (x - pivot[t]) and (x - pivot[t])^2 over its piece of row t (zero in lanes that hold nothing),
+// pivot[t] wave-uniform.  The eight sums are added up over the wave so that each lane ends with the pair of ONE row:
+// lanes exchange halves of what they hold with lane ^ 1 (even lanes keep rows 0 and 1, odd ones 2 and 3), then with
+// lane ^ 2, and the remaining pair is summed over the other four lane bits.  Lane l then holds row
+// 2 (l % 2) + (l / 2) % 2 and works out that row's record - the four records are made side by side in different
+// lanes, not one after the other in all of them - and lanes 0..7 write the 128 contiguous bytes at `rec4` (the record
+// of the first row; the rows are consecutive): half (l / 4) % 2 of their row.  Rows nrows .. 3 are not written.
+// (The pivots come by value: behind a reference the selection below turns into a load through a computed address
+// and the array into a spill.)
+__device__ __forceinline__ void write_records4(const float (&st)[8], float pivot0, float pivot1, float pivot2,
+                                               float pivot3, int C, float eps, u32x4 *__restrict__ rec4,
+                                               int nrows = 4)
+{
+    const int lane = threadIdx.x & 63;
+    const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
+    float r4[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float keep = b0 ? st[4 + i] : st[i], send = b0 ? st[i] : st[4 + i];
+        r4[i] = keep + dpp_move<0xB1>(send);                 // lane ^ 1
+    }
+    float tot[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float keep = b1 ? r4[2 + i] : r4[i], send = b1 ? r4[i] : r4[2 + i];
+        tot[i] = sum_over_lane_bits_2_to_5(keep + dpp_move<0x4E>(send));      // lane ^ 2, then the rest
+    }
+    const float pv = b0 ? (b1 ? pivot3 : pivot2) : (b1 ? pivot1 : pivot0);
+    u32x4 lo, hi;
+    row_record(pv, tot[0], tot[1], C, eps, lo, hi);
+    const int row = 2 * (lane & 1) + ((lane >> 1) & 1), half = (lane >> 2) & 1;
+    if (lane < 8 && row < nrows) rec4[row * 2 + half] = half ? hi : lo;
+}
+
 __device__ __forceinline__ int64_t live_rows(const int64_t *rows_dev, int64_t rows)
 {
     if (rows_dev == nullptr) return rows;

@@ -822,31 +822,6 @@ __global__ __launch_bounds__(256) void decompress_ln_kernel(const T *__restrict_
 // router sums them, and finishes with the router's Linear + argmax on the NEXT block's gate weights: the indices
 // and logits it leaves are bit for bit those of router_kernel run on `out`, without a second pass over the tokens.
 // The group of a sample's first region also scatters the sample's extra tokens.
-// Statistics record of one stored row from the group's sums of (x - pivot) and (x - pivot)^2, the pivot being a value
-// of the row itself (no cancellation however far the row's mean is from zero).  Values are wave-uniform.
-// Lane exchanges of the record sums below: the value of the lane whose number differs in one bit.
-template <int CTRL> __device__ __forceinline__ float dpp_move(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-// v summed over the lanes that differ in bits 2..5 of the lane number (16 of them), returned in each of them
-__device__ __forceinline__ float sum_over_lane_bits_2_to_5(float v)
-{
-    v += dpp_move<0x141>(dpp_move<0x1B>(v));      // lane ^ 4: the quad reversed, then the half row mirrored
-    v += dpp_move<0x128>(v);                      // lane ^ 8: the row rotated by eight
-    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);        // lane ^ 16: odd rows swapped with even rows
-    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);     // lane ^ 32: the halves swapped
-}
-
-__device__ __forceinline__ void row_record(float pivot, float s1, float s2, int C, float eps, u32x4 &lo, u32x4 &hi)
-{
-    const float m = s1 / (float)C;
-    const float var = fmaxf(s2 / (float)C - m * m, 0.f);
-    ln_record(pivot + m, sqrtf(var + eps), lo, hi);
-}
-
 // STAT (one wave per region, all 64 lanes present, `act` false for lanes past the row): also writes the
 // statistics records of the 16 stored rows, `rec` pointing at the record of the region's first token.
 template <typename T, int PS, bool SUB, bool STAT = false>
@@ -921,32 +896,7 @@ __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T
                 st[2 * dx + 1] = act ? q : 0.f;
             }
         }
-        if constexpr (STAT) {
-            // The eight sums (two per token) are added up over the wave so that each lane ends with the pair of ONE
-            // token: lanes exchange halves of what they hold with lane ^ 1 (even lanes keep tokens 0 and 1, odd ones
-            // 2 and 3), then with lane ^ 2, and the remaining pair is summed over the other four lane bits.  Lane l
-            // then holds token 2 (l % 2) + (l / 2) % 2, works out that token's record - the four records are made side
-            // by side in different lanes, not one after the other in all of them - and lanes 0..7 write the 128
-            // contiguous bytes: half (l / 4) % 2 of their token.
-            const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
-            float r4[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float keep = b0 ? st[4 + i] : st[i], send = b0 ? st[i] : st[4 + i];
-                r4[i] = keep + dpp_move<0xB1>(send);                 // lane ^ 1
-            }
-            float tot[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const float keep = b1 ? r4[2 + i] : r4[i], send = b1 ? r4[i] : r4[2 + i];
-                tot[i] = sum_over_lane_bits_2_to_5(keep + dpp_move<0x4E>(send));      // lane ^ 2, then the rest
-            }
-            const float pv = b0 ? (b1 ? pivot[3] : pivot[2]) : (b1 ? pivot[1] : pivot[0]);
-            u32x4 lo, hi;
-            row_record(pv, tot[0], tot[1], C, eps, lo, hi);
-            const int tok = 2 * (lane & 1) + ((lane >> 1) & 1), half = (lane >> 2) & 1;
-            if (lane < 8) rec[((int64_t)dy * W + tok) * 2 + half] = half ? hi : lo;
-        }
+        if constexpr (STAT) write_records4(st, pivot[0], pivot[1], pivot[2], pivot[3], C, eps, rec + (int64_t)dy * W * 2);
     }
 }
 
@@ -956,7 +906,8 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
     const int64_t *__restrict__ splits, const int64_t *__restrict__ offsets, const T *__restrict__ ref,
     T *__restrict__ out, const T *__restrict__ weight, const T *__restrict__ bias, T *__restrict__ gate,
     int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2,
-    u32x4 *__restrict__ records = nullptr, float eps = 0.f)
+    u32x4 *__restrict__ records = nullptr, float eps = 0.f, const int64_t *__restrict__ next_splits = nullptr,
+    uint8_t *__restrict__ next_counts = nullptr)
 {
     static_assert(!STAT || (GS == WAVE && std::is_same<T, bf16_t>::value), "records: one wave per region, bf16 rows");
     constexpr int VEC = Elem<T>::VEC;
@@ -1074,7 +1025,13 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
             }
         }
     }
-    if (lane == 0) indices[region] = best_s;
+    if (lane == 0) {
+        indices[region] = best_s;
+        if (next_counts != nullptr) {        // queries the next block takes from this region: its split, squared
+            const int ps2 = (int)next_splits[best_s];
+            next_counts[region] = (uint8_t)(ps2 * ps2);
+        }
+    }
 }
 
 // --------------------------------------------------------------- layernorm
@@ -1462,9 +1419,12 @@ extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const
 extern "C" int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices,
                                        const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
                                        const void *next_weight, const void *next_bias, void *next_gate,
-                                       int64_t *next_indices, void *out_records, float records_eps, int B, int H,
-                                       int W, int C, int extra, int R, int S, int S2, int dtype, void *stream)
+                                       int64_t *next_indices, void *out_records, float records_eps,
+                                       const int64_t *next_splits, uint8_t *next_counts, int B, int H, int W, int C,
+                                       int extra, int R, int S, int S2, int dtype, void *stream)
 {
+    VT_REQUIRE(next_counts == nullptr || (next_splits != nullptr && next_indices != nullptr), VTDGE_ERR_ARG,
+               "decompress_router: the next block's query counts need its router and its splits");
     VT_REQUIRE(in && cur_indices && splits && offsets && ref && out, VTDGE_ERR_ARG, "decompress_router: NULL operand");
     VT_REQUIRE((next_weight == nullptr) == (next_bias == nullptr) && (next_weight == nullptr) == (next_indices == nullptr),
                VTDGE_ERR_ARG, "decompress_router: the next router needs weight, bias and indices together");
@@ -1489,7 +1449,7 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
     decompress_route_kernel<bf16_t, WAVE, SUBF, true><<<grid, block, 0, st>>>(                                       \
         (const bf16_t *)in, (const bf16_t *)sub, cur_indices, splits, offsets, (const bf16_t *)ref, (bf16_t *)out,   \
         (const bf16_t *)next_weight, (const bf16_t *)next_bias, (bf16_t *)next_gate, next_indices, B, H, W, C, extra, \
-        S, S2, (u32x4 *)out_records, records_eps)
+        S, S2, (u32x4 *)out_records, records_eps, next_splits, next_counts)
         if (sub) VT_STAT(true); else VT_STAT(false);
 #undef VT_STAT
         return check_launch("decompress_router");
@@ -1497,7 +1457,8 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
 #define VT_LAUNCH2(T, GS, SUBF)                                                                                    \
     decompress_route_kernel<T, GS, SUBF><<<grid, block, 0, st>>>(                                                  \
         (const T *)in, (const T *)sub, cur_indices, splits, offsets, (const T *)ref, (T *)out,                     \
-        (const T *)next_weight, (const T *)next_bias, (T *)next_gate, next_indices, B, H, W, C, extra, S, S2)
+        (const T *)next_weight, (const T *)next_bias, (T *)next_gate, next_indices, B, H, W, C, extra, S, S2,      \
+        nullptr, 0.f, next_splits, next_counts)
 #define VT_LAUNCH(T, GS) do { if (sub) VT_LAUNCH2(T, GS, true); else VT_LAUNCH2(T, GS, false); } while (0)
 #define VT_GROUP(T) \
     do { if (gs == 64) VT_LAUNCH(T, 64); else if (gs == 32) VT_LAUNCH(T, 32); else if (gs == 16) VT_LAUNCH(T, 16); \

@@ -43,6 +43,24 @@ FUSE_PATCH_EMBED = True
 # B N tokens whatever the router decides, the routing chain only the queries, so in most layers the Linear is the
 # longer of the two (measured: +0.5 % end to end against the Linear on the second stream).
 ROUTING_ON_SIDE = True
+# The q Linear issued behind the join, on the caller's stream, instead of at the end of the routing chain: the chain
+# (index->patch, compress) then ends before the key/value Linear does, and the wait across queues that attention would
+# otherwise make for the chain's last kernel is over by the time the caller's stream reaches it.
+Q_AFTER_JOIN = True
+# index->patch and compress as one kernel that works by region (`vtdge_compress_regions`): the routing chain loses
+# its first, latency-bound kernel, and with FOLD_NORMS the q Linear takes norm1 folded in (statistics records of the
+# packed rows instead of their normalised copy).  Taken where the kernel applies (regions of 4, rows of 264 to 512
+# channels in bf16).
+REGION_COMPRESS = True
+# A kernel of the routing chain can only run beside the key/value Linear where that leaves it registers: the
+# weight-stationary Linear fills every SIMD with two waves of 216 registers, so `compress` gets one wave per SIMD and
+# finishes 10 - 20 us after the Linear instead of under it, and the fork and the join of the two streams cost 5 and
+# 9.5 us of idle queue each.  Where both kernels apply (the 384-channel bf16 models) the block therefore runs on ONE
+# stream, routing chain first (it reads the tokens the scatter-back has just written): measured +1 % end to end
+# against two streams, and no second queue in the captured graph.
+SERIAL_BESIDE_WEIGHT_STATIONARY = True
+ROUTING_FIRST = True
+Q_BEFORE_KV = True
 
 
 def _side_stream(device, slot=0):
@@ -66,7 +84,8 @@ def prepare(model):
             ops.packed_weight(mod.weight)
         # a block's LayerNorms folded into the Linears behind them (see FOLD_NORMS)
         if FOLD_NORMS and all(hasattr(mod, name) for name in ("norm1", "norm2", "attn", "mlp")):
-            for norm, lin in ((mod.norm1, getattr(mod.attn, "kv", None)), (mod.norm2, getattr(mod.mlp, "fc1", None))):
+            for norm, lin in ((mod.norm1, getattr(mod.attn, "kv", None)), (mod.norm1, getattr(mod.attn, "q", None)),
+                              (mod.norm2, getattr(mod.mlp, "fc1", None))):
                 w = getattr(lin, "weight", None)
                 if (w is not None and w.is_cuda and w.dtype == torch.bfloat16 and w.shape[1] == 384
                         and w.shape[0] % 384 == 0 and w.shape[0] <= 3072):
@@ -138,9 +157,13 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
     routed = carry.get("routed") if gate is None else None
 
     n1, n2 = block.norm1, block.norm2
-    overlap = overlap and OVERLAP
+    fold1 = (FOLD_NORMS and x_ln is None and getattr(attn, "sr_ratio", 1) <= 1
+             and ops.fits_linear_layernorm(x, attn.kv.weight))
+    use_regions = REGION_COMPRESS and ops.fits_compress_regions(x, H, W, R, dge.router.split_sizes)
+    overlap = overlap and OVERLAP and not (SERIAL_BESIDE_WEIGHT_STATIONARY and fold1 and use_regions)
     main = torch.cuda.current_stream(x.device)
     side = _side_stream(x.device, main.cuda_stream) if overlap else main
+    swap = overlap and ROUTING_ON_SIDE
 
     fuse_rn = (FUSE_ROUTER_NORM and gate is None and routed is None and x_ln is None
                and ops.fits_router_layernorm(x, R))
@@ -148,47 +171,82 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         gate, indices, x_ln = ops.router_layernorm(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R,
                                                    n1.weight, n1.bias, n1.eps)
 
-    # key/value chain (one of the two streams, see ROUTING_ON_SIDE)
-    if overlap:
-        side.wait_stream(main)
-    fold1 = (FOLD_NORMS and x_ln is None and getattr(attn, "sr_ratio", 1) <= 1
-             and ops.fits_linear_layernorm(x, attn.kv.weight))
-    swap = overlap and ROUTING_ON_SIDE
-    with torch.cuda.stream(main if swap else side):
+    def kv_chain():
+        nonlocal x_ln
         if fold1:
             rec1 = carry.get("x_stats")
             if rec1 is None:
                 rec1 = ops.layernorm_stats(x, n1.eps)
-            kv_src = x
-            kv = ops.linear_layernorm(x, rec1, attn.kv.weight, attn.kv.bias, n1.weight, n1.bias)
-        else:
-            if x_ln is None:
-                x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
-            kv_src = _key_value_source(attn, x_ln, H, W, extra)
-            kv = ops.linear(kv_src, attn.kv.weight, attn.kv.bias)             # [B, n, 2C] = [B, n, 2, h, d]
+            return x, ops.linear_layernorm(x, rec1, attn.kv.weight, attn.kv.bias, n1.weight, n1.bias)
+        if x_ln is None:
+            x_ln = ops.layernorm(x, n1.weight, n1.bias, n1.eps)
+        src = _key_value_source(attn, x_ln, H, W, extra)
+        return src, ops.linear(src, attn.kv.weight, attn.kv.bias)             # [B, n, 2C] = [B, n, 2, h, d]
 
-    # routing chain (the other stream)
-    with torch.cuda.stream(side if swap else main):
+    cap = B * N
+
+    def routing_chain():
+        """-> (gate, indices, patches, offsets, lengths, comp, LayerNorm(comp) or None, records of comp or None)"""
+        g, idx = gate, None
         if routed is not None:
-            gate, indices = routed
-        elif not fuse_rn:
-            if gate is None:
-                gate, indices = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
-            else:
-                indices = gate.argmax(dim=-1)
-        cap = B * N
-        patches, offsets, lengths = ops.index_to_patch(indices, dge.splits, R, extra, capacity=cap)
-        rows_dev = offsets[B:]
-        comp, comp_ln = ops.compress(x, patches, W, extra, rows_dev=rows_dev, rows=cap, ln_weight=n1.weight,
-                                     ln_bias=n1.bias, ln_eps=n1.eps)
-        q = ops.linear(comp_ln, attn.q.weight, attn.q.bias, rows_dev=rows_dev)
+            g, idx = routed
+        elif fuse_rn:
+            idx = indices
+        elif g is None:
+            g, idx = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
+        else:
+            idx = g.argmax(dim=-1)
+        if use_regions:
+            # index->patch and compress in one kernel, by region; with the folded norm1 -> q it leaves the statistics
+            # records of the packed rows instead of their normalised copy
+            foldq = FOLD_NORMS and ops.fits_linear_layernorm(x, attn.q.weight)
+            cmp_, rec, pat, off, lens = ops.compress_regions(
+                x, idx, dge.splits, H, W, R, counts=carry.get("counts") if routed is not None else None,
+                stats_eps=n1.eps if foldq else None, capacity=cap)
+            ln = None if foldq else ops.layernorm(cmp_, n1.weight, n1.bias, n1.eps, rows_dev=off[B:])
+            return g, idx, pat, off, lens, cmp_, ln, rec
+        pat, off, lens = ops.index_to_patch(idx, dge.splits, R, extra, capacity=cap)
+        cmp_, ln = ops.compress(x, pat, W, extra, rows_dev=off[B:], rows=cap, ln_weight=n1.weight, ln_bias=n1.bias,
+                                ln_eps=n1.eps)
+        return g, idx, pat, off, lens, cmp_, ln, None
 
+    def q_linear():
+        if comp_rec is not None:
+            return ops.linear_layernorm(comp, comp_rec, attn.q.weight, attn.q.bias, n1.weight, n1.bias,
+                                        rows_dev=rows_dev)
+        return ops.linear(comp_ln, attn.q.weight, attn.q.bias, rows_dev=rows_dev)
+
+    q = None
     if overlap:
+        # the two chains side by side on two streams, joined before attention
+        side.wait_stream(main)
+        with torch.cuda.stream(main if swap else side):
+            kv_src, kv = kv_chain()
+        with torch.cuda.stream(side if swap else main):
+            gate, indices, patches, offsets, lengths, comp, comp_ln, comp_rec = routing_chain()
+            rows_dev = offsets[B:]
+            if not Q_AFTER_JOIN:
+                q = q_linear()
         main.wait_stream(side)
-        crossing = (gate, indices, patches, offsets, lengths, comp, comp_ln, q) if swap else (x_ln, kv_src, kv)
+        crossing = ((gate, indices, patches, offsets, lengths, comp, comp_ln, comp_rec, q) if swap
+                    else (x_ln, kv_src, kv))
         for t in crossing:
             if t is not None:
                 t.record_stream(main)    # allocated on the side stream, consumed (and released) on the caller's
+        if q is None:
+            q = q_linear()
+    else:
+        # one stream: the routing chain, then the two Linears
+        if not ROUTING_FIRST:
+            kv_src, kv = kv_chain()
+        gate, indices, patches, offsets, lengths, comp, comp_ln, comp_rec = routing_chain()
+        rows_dev = offsets[B:]
+        if Q_BEFORE_KV:
+            q = q_linear()
+        if ROUTING_FIRST:
+            kv_src, kv = kv_chain()
+        if q is None:
+            q = q_linear()
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
     fold2 = FOLD_NORMS and ops.fits_linear_layernorm(o, mlp.fc1.weight)
     if fold2 and ops.fits_linear_stats(o, attn.proj.weight):
@@ -215,13 +273,17 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         nattn = next_block.attn
         want_stats = (FOLD_NORMS and getattr(nattn, "sr_ratio", 1) <= 1 and ops.fits_scatter_stats(x)
                       and ops.fits_linear_layernorm(x, nattn.kv.weight))
+        want_counts = REGION_COMPRESS and ops.fits_compress_regions(x, H, W, 4, nxt.router.split_sizes)
         res = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
                                     next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias,
-                                    stats_eps=next_block.norm1.eps if want_stats else None)
+                                    stats_eps=next_block.norm1.eps if want_stats else None,
+                                    next_splits=nxt.splits if want_counts else None)
         out, ngate, nidx = res[:3]
         handed["routed"] = (ngate, nidx)
         if want_stats:
             handed["x_stats"] = res[3]
+        if want_counts:
+            handed["counts"] = res[-1]
     else:
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 

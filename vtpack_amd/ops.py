@@ -174,12 +174,71 @@ def decompress_layernorm(inp, patches, reference, width, num_extra_tokens, ln_we
     return out, ln_out
 
 
+def region_counts_buffer(B, regions, device):
+    """An uninitialised uint8 buffer for the per-region query counts `decompress_router` leaves for
+    `compress_regions`, padded so that the reader's 16-byte loads stay inside it."""
+    return torch.empty((-(-(B * regions) // 16) * 16,), dtype=torch.uint8, device=device)
+
+
+def fits_compress_regions(x, H, W, region_size, split_sizes):
+    """Whether `compress_regions` has a kernel: regions of 4 x 4 tokens split 1, 2 or 4 ways, a row of at most 64
+    16-byte vectors (and more than 32: narrower rows are better served by the row-wise kernels, which give several
+    rows to a wave), at most 65536 regions."""
+    if x.dim() != 3 or x.dtype not in (torch.float32, torch.bfloat16) or region_size != 4:
+        return False
+    B, N, C = x.shape
+    nvec = C * x.element_size() // 16
+    return (x.is_cuda and H % 4 == 0 and W % 4 == 0 and N >= H * W and N - H * W <= 64
+            and (C * x.element_size()) % 16 == 0 and 32 < nvec <= 64
+            and set(int(s) for s in split_sizes) <= {1, 2, 4}
+            and B * (H // 4) * (W // 4) <= 65536 and B * N < (1 << 24))
+
+
+def compress_regions(x, indices, splits, H, W, region_size=4, counts=None, stats_eps=None, capacity=None,
+                     want_patches=True):
+    """index_to_patch and compress in one kernel, by region: x [B, extra + H*W, C] and the gate indices [B, Hr, Wr]
+    -> (comp [capacity, C], records or None, patches or None, offsets [B+1], lengths [B]).  `counts` is the uint8
+    buffer a `decompress_router(..., next_splits=...)` has filled for these indices (optional: the kernel otherwise
+    works the counts out from the indices); with `stats_eps` (bf16) the statistics records of the rows of comp are
+    written for a `linear_layernorm` that takes comp next.  comp, patches, offsets and lengths equal those of
+    `index_to_patch` + `compress` bit for bit.  vtpack/layers/dge.py:76-79."""
+    _need_gpu(x, indices, splits, counts)
+    x, indices, splits = _contig(x), _contig(indices), _contig(splits)
+    if indices.dtype != torch.int64 or splits.dtype != torch.int64 or indices.dim() != 3:
+        raise TypeError("indices must be int64 [B, Hr, Wr] and splits int64")
+    B, N, C = x.shape
+    extra = N - H * W
+    if extra < 0 or H % region_size or W % region_size or tuple(indices.shape) != (B, H // region_size, W // region_size):
+        raise ValueError(f"gate indices {tuple(indices.shape)} do not match a {H}x{W} grid of regions of {region_size}")
+    regions = (H // region_size) * (W // region_size)
+    if counts is not None and (counts.dtype != torch.uint8 or counts.numel() < -(-(B * regions) // 16) * 16):
+        raise ValueError("counts must be a uint8 buffer from region_counts_buffer")
+    if stats_eps is not None and x.dtype != torch.bfloat16:
+        raise TypeError("compress_regions: records exist for bfloat16 rows only")
+    if capacity is None:
+        capacity = B * N
+    if capacity < B * N:
+        raise ValueError("compress_regions writes without bounds checks on comp: capacity must be at least B * N")
+    comp = torch.empty((capacity, C), dtype=x.dtype, device=x.device)
+    rec = torch.empty((capacity, 16), dtype=torch.bfloat16, device=x.device) if stats_eps is not None else None
+    patches = torch.empty((capacity, 4), dtype=torch.int64, device=x.device) if want_patches else None
+    offsets = torch.empty((B + 1,), dtype=torch.int64, device=x.device)
+    lengths = torch.empty((B,), dtype=torch.int64, device=x.device)
+    call("vtdge_compress_regions", ptr(x), ptr(indices), ptr(splits), ptr(counts), ptr(comp), ptr(rec),
+         float(stats_eps if stats_eps is not None else 0.0), ptr(patches), capacity, ptr(offsets), ptr(lengths),
+         B, H, W, C, extra, region_size, splits.numel(), dtype_code(x), stream_ptr(),
+         tag=("compress_regions", rec is not None, C, counts is not None))
+    return comp, rec, patches, offsets, lengths
+
+
 def decompress_router(inp, indices, splits, offsets, reference, H, W, region_size, sub=None, next_weight=None,
-                      next_bias=None, want_gate=True, stats_eps=None):
+                      next_bias=None, want_gate=True, stats_eps=None, next_splits=None):
     """Scatter (inp - sub) + reference back over the tokens by region, and route the NEXT block on the result:
     -> (out, next_gate or None, next_indices or None), and with `stats_eps` (a LayerNorm's eps; bf16 rows of 264 to
-    512 channels) a fourth value: the statistics records of the rows of `out` for `linear_layernorm`.  `indices` [B, Hr, Wr] are this block's gate indices, `offsets`
-    [B+1] the prefix of its query counts.  The three outputs equal decompress(...) and router(out, next_weight,
+    512 channels) a fourth value: the statistics records of the rows of `out` for `linear_layernorm`; with `next_splits`
+    (the next block's split sizes, int64 on the device) one more at the end: the uint8 query counts of the next block's
+    regions for `compress_regions`.  `indices` [B, Hr, Wr] are this block's gate indices, `offsets` [B+1] the prefix of
+    its query counts.  The three outputs equal decompress(...) and router(out, next_weight,
     next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75."""
     _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
     inp, reference = _contig(inp), _contig(reference)
@@ -210,14 +269,20 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
     rec = None
     if stats_eps is not None:
         rec = torch.empty((B * N, 16), dtype=torch.bfloat16, device=inp.device)
+    counts = None
+    if next_splits is not None:
+        if next_weight is None or next_splits.dtype != torch.int64 or next_splits.numel() != S2:
+            raise ValueError("next_splits goes with the next router: int64, one entry per row of next_weight")
+        _need_gpu(next_splits)
+        next_splits = _contig(next_splits)
+        counts = region_counts_buffer(B, (H // region_size) * (W // region_size), inp.device)
     call("vtdge_decompress_router", ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference),
          ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), ptr(rec),
-         float(stats_eps if stats_eps is not None else 0.0), B, H, W, C, extra, region_size, S, S2,
-         dtype_code(inp), stream_ptr(),
+         float(stats_eps if stats_eps is not None else 0.0), ptr(next_splits), ptr(counts), B, H, W, C, extra,
+         region_size, S, S2, dtype_code(inp), stream_ptr(),
          tag=("decompress_router", sub is not None, next_weight is not None, C, rec is not None))
-    if stats_eps is not None:
-        return out, gate, nidx, rec
-    return out, gate, nidx
+    res = (out, gate, nidx) + ((rec,) if stats_eps is not None else ()) + ((counts,) if counts is not None else ())
+    return res
 
 
 def fits_scatter_stats(x):
