@@ -90,8 +90,12 @@ def kernel_symbol(name, tag, dt, n_keys=0):
         return f"linear_dma_kernel<{T}, {tile}, 0, true, false, 3, false, true>"
     if name == "vtdge_linear_layernorm":
         return f"linear_ws8_kernel<{1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
+    if name == "vtdge_linear_layernorm_pair":
+        return "linear_ws8_pair_kernel<0>"
     if name == "vtdge_linear_stats":
         return f"linear_ws8_kernel<0, {b(tag[1])}, {b(tag[2])}, false, true>"
+    if name == "vtdge_compress_regions":
+        return f"compress_regions_kernel<{T}, {b(tag[1])}>"
     gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
     if name == "vtdge_layernorm_stats":
         nv = tag[2] * esz // 16
@@ -165,6 +169,17 @@ def algorithmic_work(name, tag, esz, geo):
         M = L if packed else rows
         # raw rows, their 32-byte records, the folded weights and their records, the output
         return "mfma", 2.0 * M * Nn * K, (M * K + Nn * K + M * Nn) * esz + 32 * (M + Nn)
+    if name == "vtdge_linear_layernorm_pair":
+        # two Linears: (rows, N, packed) each; K is the width of the tokens
+        flops = byts = 0.0
+        for rows, Nn, packed in (tag[1:4], tag[4:7]):
+            M = L if packed else rows
+            flops += 2.0 * M * Nn * C
+            byts += (M * C + Nn * C + M * Nn) * esz + 32 * (M + Nn)
+        return "mfma", flops, byts
+    if name == "vtdge_compress_regions":
+        # every token once, the gate indices and count bytes, every query once with its record and descriptor
+        return "hbm", B * N * C * esz + 9 * B * geo["regions"] + L * C * esz + (32 * L if tag[1] else 0) + 32 * L
     if name == "vtdge_layernorm_stats":
         rows = L if tag[1] != B * N else tag[1]
         return "hbm", rows * tag[2] * esz + 32.0 * rows

@@ -259,6 +259,18 @@ int vtdge_linear_layernorm(const void *A, int64_t lda, const void *row_records, 
                            const void *packed, const void *col_records, void *out, int64_t ldo,
                            const int64_t *rows_dev, int64_t rows, int N, int K, int act, int dtype, void *stream);
 
+/* Two vtdge_linear_layernorm calls without activation as ONE launch: norm1 -> kv on all tokens and norm1 -> q on the
+ * packed queries (vtpack/models/dge/deit_dge.py:127 with :73 and :72), which the reference issues one after the
+ * other.  The workgroups are dealt out between the two in proportion to their live rows (read on the device), so
+ * the smaller one no longer runs a few tiles per workgroup behind the fixed cost of a launch of its own.  Operands
+ * with suffix 0 and 1 as in vtdge_linear_layernorm, same K; results are bit-identical to the two separate calls. */
+int vtdge_linear_layernorm_pair(const void *A0, int64_t lda0, const void *row_records0, const void *W_folded0,
+                                const void *packed0, const void *col_records0, void *out0, int64_t ldo0,
+                                const int64_t *rows_dev0, int64_t rows0, int N0, const void *A1, int64_t lda1,
+                                const void *row_records1, const void *W_folded1, const void *packed1,
+                                const void *col_records1, void *out1, int64_t ldo1, const int64_t *rows_dev1,
+                                int64_t rows1, int N1, int K, int dtype, void *stream);
+
 /* Sparse attention of packed queries against each sample's full K/V:
  *   out[rows of sample i, head a] = softmax(scale * Q_i,a K_i,a^T) V_i,a
  * Replaces batched_sparse_attention_forward

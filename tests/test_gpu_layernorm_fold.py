@@ -205,6 +205,32 @@ def test_operand_checks(dev):
     assert not ops.fits_linear_layernorm(x, torch.zeros(100, C, dtype=torch.bfloat16, device=dev))
 
 
+@pytest.mark.parametrize("live1", [None, 0, 1, 31, 33, 700, 2599, 11000, 60000])
+@pytest.mark.parametrize("M0,N0,N1", [(65792, 768, 384), (2600, 768, 384), (4097, 384, 1536)])
+def test_two_linears_in_one_launch(dev, M0, N0, N1, live1):
+    """norm1 -> kv on all tokens and norm1 -> q on the packed rows as one launch whose workgroups are shared out by
+    the live row counts: the same bytes as the two separate launches, whatever the split."""
+    from vtpack_amd import ops
+    M1 = max(M0, 2048 if live1 is None else live1)
+    x0 = rows_like_tokens(M0, 31, 1.0, dev)
+    x1 = rows_like_tokens(M1, 32, 0.5, dev)
+    w0, b0, gamma, beta = layer(N0, 33, dev)
+    w1, b1, _, _ = layer(N1, 34, dev)
+    rows_dev1 = None if live1 is None else torch.tensor([live1], dtype=torch.int64, device=dev)
+    L1 = M1 if live1 is None else live1
+    rec0 = ops.layernorm_stats(x0, EPS)
+    rec1 = ops.layernorm_stats(x1, EPS, rows_dev=rows_dev1)
+    want0 = ops.linear_layernorm(x0, rec0, w0, b0, gamma, beta)
+    want1 = ops.linear_layernorm(x1, rec1, w1, b1, gamma, beta, rows_dev=rows_dev1)
+    got0, got1 = ops.linear_layernorm_pair(x0, rec0, w0, b0, x1, rec1, w1, b1, gamma, beta, rows_dev1=rows_dev1)
+    assert torch.equal(got0, want0)
+    assert torch.equal(got1[:L1], want1[:L1])
+    # the other way round, and the first one short
+    rows_dev0 = torch.tensor([min(M0, 777)], dtype=torch.int64, device=dev)
+    a, b = ops.linear_layernorm_pair(x1, rec1, w1, b1, x0, rec0, w0, b0, gamma, beta, rows_dev0=rows_dev1, rows_dev1=rows_dev0)
+    assert torch.equal(a[:L1], want1[:L1]) and torch.equal(b[:min(M0, 777)], want0[:min(M0, 777)])
+
+
 # ----------------------------------------------------------------------------- records from the producing kernels
 @pytest.mark.parametrize("live", [None, 0, 17, 33, 64, 2599])
 @pytest.mark.parametrize("has_bias,has_res", [(True, True), (True, False), (False, True), (False, False)])
@@ -338,7 +364,8 @@ def test_model_with_and_without_folded_norms(dev):
     (on, len_on, names_on), (off, len_off, names_off) = runs[True], runs[False]
     assert names_off.count("vtdge_layernorm") == 37 and names_off.count("vtdge_linear_layernorm") == 0
     assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 1
-    assert names_on.count("vtdge_linear_layernorm") == 36 and names_on.count("vtdge_linear_stats") == 12
+    assert names_on.count("vtdge_linear_layernorm") == 12 and names_on.count("vtdge_linear_layernorm_pair") == 12
+    assert names_on.count("vtdge_linear_stats") == 12
     assert torch.equal(len_on[0], len_off[0])
     if all(torch.equal(a, b) for a, b in zip(len_on, len_off)):
         assert abs_err(on, off) <= 2 * BF16_ABS

@@ -46,6 +46,8 @@ SIGNATURES = {
     "vtdge_layernorm_stats": [_p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_layernorm_fold": [_p, _p, _p, _p, _i, _i, _i, _p, _p, _p],
     "vtdge_linear_layernorm": [_p, _l, _p, _p, _p, _p, _p, _l, _p, _l, _i, _i, _i, _i, _p],
+    "vtdge_linear_layernorm_pair": [_p, _l, _p, _p, _p, _p, _p, _l, _p, _l, _i, _p, _l, _p, _p, _p, _p, _p, _l, _p, _l,
+                                    _i, _i, _i, _p],
     "vtdge_sparse_attention": [_p, _l, _l, _p, _p, _l, _l, _l, _p, _p, _l, _l, _i, _i, _i, _i, _i, _f, _i, _p],
     "vtdge_batched_sparse_gemm": [_p, _p, _p, _p, _p, _i, _i, _l, _i, _l, _i, _i, _i, _l, _l, _l, _i, _p],
 }

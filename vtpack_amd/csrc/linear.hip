@@ -205,6 +205,11 @@ bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, i
 int launch_linear_ws8(const void *A, int64_t lda, const void *W, const void *Wp, const void *bias, const void *res,
                       int64_t ldr, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N, int act,
                       hipStream_t st);
+int launch_linear_ws8_ln_pair(const void *A0, int64_t lda0, const void *lnrec0, const void *Wf0, const void *Wfp0,
+                              const void *lnw0, void *out0, int64_t ldo0, const int64_t *rows_dev0, int64_t rows0,
+                              int N0, const void *A1, int64_t lda1, const void *lnrec1, const void *Wf1,
+                              const void *Wfp1, const void *lnw1, void *out1, int64_t ldo1, const int64_t *rows_dev1,
+                              int64_t rows1, int N1, hipStream_t st);
 int launch_linear_ws8_ln(const void *A, int64_t lda, const void *lnrec, const void *Wf, const void *Wfp,
                          const void *lnw, void *out, int64_t ldo, const int64_t *rows_dev, int64_t rows, int N,
                          int act, hipStream_t st);
@@ -345,6 +350,36 @@ extern "C" int vtdge_linear_layernorm(const void *A, int64_t lda, const void *ro
                "(rows=%lld N=%d K=%d dtype=%d)", (long long)rows, N, K, dtype);
     return launch_linear_ws8_ln(A, lda, row_records, W_folded, packed, col_records, out, ldo, rows_dev, rows, N, act,
                                 (hipStream_t)stream);
+}
+
+extern "C" int vtdge_linear_layernorm_pair(const void *A0, int64_t lda0, const void *row_records0, const void *W_folded0,
+                                           const void *packed0, const void *col_records0, void *out0, int64_t ldo0,
+                                           const int64_t *rows_dev0, int64_t rows0, int N0, const void *A1,
+                                           int64_t lda1, const void *row_records1, const void *W_folded1,
+                                           const void *packed1, const void *col_records1, void *out1, int64_t ldo1,
+                                           const int64_t *rows_dev1, int64_t rows1, int N1, int K, int dtype,
+                                           void *stream)
+{
+    VT_REQUIRE(A0 && row_records0 && W_folded0 && col_records0 && out0 && A1 && row_records1 && W_folded1 &&
+                   col_records1 && out1,
+               VTDGE_ERR_ARG, "linear_layernorm_pair: NULL operand");
+    VT_REQUIRE(rows0 >= 0 && rows1 >= 0 && N0 > 0 && N1 > 0 && K > 0, VTDGE_ERR_ARG, "linear_layernorm_pair: bad sizes");
+    VT_REQUIRE(lda0 >= K && ldo0 >= N0 && lda1 >= K && ldo1 >= N1, VTDGE_ERR_ARG,
+               "linear_layernorm_pair: leading dim too small");
+    VT_REQUIRE((((uintptr_t)A0 | (uintptr_t)W_folded0 | (uintptr_t)packed0 | (uintptr_t)row_records0 |
+                 (uintptr_t)col_records0 | (uintptr_t)A1 | (uintptr_t)W_folded1 | (uintptr_t)packed1 |
+                 (uintptr_t)row_records1 | (uintptr_t)col_records1) & 15) == 0,
+               VTDGE_ERR_ARG, "linear_layernorm_pair: operands must be 16-byte aligned");
+    VT_REQUIRE(dtype == VTDGE_BF16 &&
+                   linear_ws_applicable(lda0, 0, ldo0, rows0, N0, K, 2, VTDGE_ACT_NONE, nullptr, nullptr, out0) &&
+                   linear_ws_applicable(lda1, 0, ldo1, rows1, N1, K, 2, VTDGE_ACT_NONE, nullptr, nullptr, out1) &&
+                   N0 / 384 + N1 / 384 <= 16,
+               VTDGE_ERR_UNSUPPORTED,
+               "linear_layernorm_pair: both Linears as vtdge_linear_layernorm takes them (bf16, K = 384, N a multiple of "
+               "384, 2048 rows or more; rows=%lld,%lld N=%d,%d K=%d)", (long long)rows0, (long long)rows1, N0, N1, K);
+    return launch_linear_ws8_ln_pair(A0, lda0, row_records0, W_folded0, packed0, col_records0, out0, ldo0, rows_dev0,
+                                     rows0, N0, A1, lda1, row_records1, W_folded1, packed1, col_records1, out1, ldo1,
+                                     rows_dev1, rows1, N1, (hipStream_t)stream);
 }
 
 extern "C" int vtdge_linear_stats(const void *A, int64_t lda, const void *W, const void *packed, const void *bias,

@@ -81,11 +81,12 @@ __device__ __forceinline__ float w8_gelu(float f)
     return f * (x * q + 0.5f);
 }
 
+// The work of one workgroup: column group g of the matrix, position p among the P workgroups of that group.
 template <int ACT, bool HAS_BIAS, bool HAS_RES, bool HAS_LN, bool HAS_STAT>
-__global__ __launch_bounds__(512) void linear_ws8_kernel(
+__device__ __forceinline__ void ws8_workgroup(
     const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
     const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
-    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp,
+    const int64_t *__restrict__ rows_dev, int64_t rows, int g, int p, int P, const u32x4 *__restrict__ Wp,
     const u32x4 *__restrict__ lnrec, const u32x4 *__restrict__ lnw, u32x4 *__restrict__ stat_out, float stat_eps)
 {
     constexpr int KB = 768;                     // bytes of one operand row
@@ -106,9 +107,6 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int g = slot % groups;                     // column group
-    const int p = xcd + 8 * (slot / groups);         // position among the P workgroups of the group
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c16 = lane & 15, kg = lane >> 4;
@@ -425,6 +423,82 @@ __global__ __launch_bounds__(512) void linear_ws8_kernel(
     }
 }
 
+template <int ACT, bool HAS_BIAS, bool HAS_RES, bool HAS_LN, bool HAS_STAT>
+__global__ __launch_bounds__(512) void linear_ws8_kernel(
+    const bf16_t *__restrict__ A, int64_t lda, const bf16_t *__restrict__ Wt, const bf16_t *__restrict__ bias,
+    const bf16_t *__restrict__ res, int64_t ldr, bf16_t *__restrict__ out, int64_t ldo,
+    const int64_t *__restrict__ rows_dev, int64_t rows, int groups, int P, const u32x4 *__restrict__ Wp,
+    const u32x4 *__restrict__ lnrec, const u32x4 *__restrict__ lnw, u32x4 *__restrict__ stat_out, float stat_eps)
+{
+    // the P workgroups of a column group are spread over the 8 XCDs (consecutive workgroup numbers go to consecutive
+    // XCDs), and the workgroups that share A tiles (same position in different groups) sit on the same XCD
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int g = slot % groups;                     // column group
+    const int p = xcd + 8 * (slot / groups);         // position among the P workgroups of the group
+    ws8_workgroup<ACT, HAS_BIAS, HAS_RES, HAS_LN, HAS_STAT>(A, lda, Wt, bias, res, ldr, out, ldo, rows_dev, rows, g, p,
+                                                            P, Wp, lnrec, lnw, stat_out, stat_eps);
+}
+
+// Two Linears with folded LayerNorms in ONE launch (the key/value projection of all tokens and the query projection
+// of the packed rows: same K, same epilogue, different operands and row counts).  Alone, the smaller of the two
+// gives every workgroup three or four tiles behind the fixed cost of fetching its strip of W; here the grid is
+// dealt out between the two in proportion to their tiles, so that every workgroup has a long run of one of them.
+// The live row counts are on the device, so every workgroup works the split out for itself (the same integers in
+// all of them): units of 8 workgroups (one per XCD), na units per column group of the first problem, nb per column
+// group of the second, na * groups_a + nb * groups_b = gridDim.x / 8, chosen to minimise the longer of the two runs.
+struct Ws8Problem {
+    const bf16_t *A;
+    int64_t lda;
+    const bf16_t *Wt;
+    bf16_t *out;
+    int64_t ldo;
+    const int64_t *rows_dev;
+    int64_t rows;
+    int groups;
+    const u32x4 *Wp, *lnrec, *lnw;
+};
+
+template <int ACT>
+__global__ __launch_bounds__(512) void linear_ws8_pair_kernel(const Ws8Problem a, const Ws8Problem b)
+{
+    const int ta = (int)((live_rows(a.rows_dev, a.rows) + 31) / 32), tb = (int)((live_rows(b.rows_dev, b.rows) + 31) / 32);
+    const int units = (int)(gridDim.x >> 3);
+    // nearest split to the proportional one, then its neighbours
+    const float wa = (float)ta * a.groups, wb = (float)tb * b.groups;
+    int na = (int)((float)units * wa / fmaxf(wa + wb, 1.f) / (float)a.groups + 0.5f);
+    int best_na = 0, best_steps = 0x7fffffff;
+#pragma unroll 1
+    for (int c = na - 1; c <= na + 1; c++) {
+        if (c < 1 || c * a.groups >= units) continue;
+        const int rem = units - c * a.groups;
+        if (rem % b.groups) continue;
+        const int nb = rem / b.groups;
+        const int sa = (ta + 8 * c - 1) / (8 * c), sb = (tb + 8 * nb - 1) / (8 * nb);
+        const int steps = sa > sb ? sa : sb;
+        if (steps < best_steps) {
+            best_steps = steps;
+            best_na = c;
+        }
+    }
+    if (best_na == 0) {                      // no neighbour fits (tiny grids, awkward group counts): first valid split
+#pragma unroll 1
+        for (int c = 1; c * a.groups < units; c++)
+            if ((units - c * a.groups) % b.groups == 0) {
+                best_na = c;
+                break;
+            }
+    }
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int slots_a = best_na * a.groups;
+    const bool first = slot < slots_a;
+    const Ws8Problem &m = first ? a : b;
+    const int s2 = first ? slot : slot - slots_a;
+    const int n_units = first ? best_na : (units - slots_a) / b.groups;
+    const int g = s2 % m.groups, p = xcd + 8 * (s2 / m.groups);
+    ws8_workgroup<ACT, false, false, true, false>(m.A, m.lda, m.Wt, nullptr, nullptr, 0, m.out, m.ldo, m.rows_dev, m.rows, g,
+                                                  p, 8 * n_units, m.Wp, m.lnrec, m.lnw, nullptr, 0.f);
+}
+
 // ----------------------------------------------------------------------------- host
 bool linear_ws_applicable(int64_t lda, int64_t ldr, int64_t ldo, int64_t rows, int N, int K, int esz, int act,
                           const void *bias, const void *res, const void *out)
@@ -494,6 +568,27 @@ int launch_linear_ws8_ln(const void *A, int64_t lda, const void *lnrec, const vo
                                                                   rows_dev, rows, N, st, lnrec, lnw, nullptr, 0.f);
     return go_ws8<VTDGE_ACT_NONE, false, false, true, false>(A, lda, Wf, Wfp, nullptr, nullptr, 0, out, ldo, rows_dev,
                                                               rows, N, st, lnrec, lnw, nullptr, 0.f);
+}
+
+// two such Linears in one launch (see linear_ws8_pair_kernel)
+int launch_linear_ws8_ln_pair(const void *A0, int64_t lda0, const void *lnrec0, const void *Wf0, const void *Wfp0,
+                              const void *lnw0, void *out0, int64_t ldo0, const int64_t *rows_dev0, int64_t rows0,
+                              int N0, const void *A1, int64_t lda1, const void *lnrec1, const void *Wf1,
+                              const void *Wfp1, const void *lnw1, void *out1, int64_t ldo1, const int64_t *rows_dev1,
+                              int64_t rows1, int N1, hipStream_t st)
+{
+    constexpr size_t lds = 4 * 32 * 768 + 4 * 1024;
+    auto kern = linear_ws8_pair_kernel<VTDGE_ACT_NONE>;
+    VT_RESERVE_LDS(kern, lds, "linear");
+    const Ws8Problem a = {(const bf16_t *)A0, lda0, (const bf16_t *)Wf0, (bf16_t *)out0, ldo0, rows_dev0, rows0, N0 / 384,
+                          (const u32x4 *)Wfp0, (const u32x4 *)lnrec0, (const u32x4 *)lnw0};
+    const Ws8Problem b = {(const bf16_t *)A1, lda1, (const bf16_t *)Wf1, (bf16_t *)out1, ldo1, rows_dev1, rows1, N1 / 384,
+                          (const u32x4 *)Wfp1, (const u32x4 *)lnrec1, (const u32x4 *)lnw1};
+    // one workgroup per CU in units of 8 (one per XCD); at least one unit per column group of either problem
+    int units = compute_units() / 8;
+    if (units < a.groups + b.groups) units = a.groups + b.groups;
+    kern<<<dim3((unsigned)(units * 8)), dim3(512), lds, st>>>(a, b);
+    return check_launch("linear");
 }
 
 // out = A W^T + bias + residual for N = 384, with the statistics records of the rows of out

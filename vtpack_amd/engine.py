@@ -61,6 +61,10 @@ REGION_COMPRESS = True
 SERIAL_BESIDE_WEIGHT_STATIONARY = True
 ROUTING_FIRST = True
 Q_BEFORE_KV = True
+# On one stream the key/value Linear and the q Linear (both with norm1 folded in) go out as ONE launch
+# (`vtdge_linear_layernorm_pair`): alone the q Linear has three or four tiles per workgroup behind the fixed cost of
+# fetching its weights.
+PAIR_KV_Q = True
 
 
 def _side_stream(device, slot=0):
@@ -241,12 +245,21 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
             kv_src, kv = kv_chain()
         gate, indices, patches, offsets, lengths, comp, comp_ln, comp_rec = routing_chain()
         rows_dev = offsets[B:]
-        if Q_BEFORE_KV:
-            q = q_linear()
-        if ROUTING_FIRST:
-            kv_src, kv = kv_chain()
-        if q is None:
-            q = q_linear()
+        if PAIR_KV_Q and ROUTING_FIRST and fold1 and comp_rec is not None:
+            # the key/value and the query projection as one launch, the grid shared out by their live rows
+            rec1 = carry.get("x_stats")
+            if rec1 is None:
+                rec1 = ops.layernorm_stats(x, n1.eps)
+            kv_src = x
+            kv, q = ops.linear_layernorm_pair(x, rec1, attn.kv.weight, attn.kv.bias, comp, comp_rec, attn.q.weight,
+                                              attn.q.bias, n1.weight, n1.bias, rows_dev1=rows_dev)
+        else:
+            if Q_BEFORE_KV:
+                q = q_linear()
+            if ROUTING_FIRST:
+                kv_src, kv = kv_chain()
+            if q is None:
+                q = q_linear()
     o = ops.sparse_attention(q, kv[:, :, :C], kv[:, :, C:], offsets, attn.scale, attn.num_heads, N)
     fold2 = FOLD_NORMS and ops.fits_linear_layernorm(o, mlp.fc1.weight)
     if fold2 and ops.fits_linear_stats(o, attn.proj.weight):

@@ -575,6 +575,33 @@ def linear_layernorm(a, records, weight, bias, ln_weight, ln_bias, act="none", r
     return out
 
 
+def linear_layernorm_pair(a0, records0, weight0, bias0, a1, records1, weight1, bias1, ln_weight, ln_bias,
+                          rows_dev0=None, rows_dev1=None):
+    """(linear_layernorm(a0, records0, weight0, bias0, ...), linear_layernorm(a1, records1, weight1, bias1, ...)) with
+    the same LayerNorm weights, as one launch whose workgroups are shared out between the two by their live rows:
+    norm1 -> kv on the tokens and norm1 -> q on the packed queries.  Same bits as the two calls."""
+    _need_gpu(a0, a1, weight0, weight1, bias0, bias1, ln_weight, ln_bias, records0, records1)
+    outs, args, shapes = [], [], ()
+    for a, rec, w, b, rd in ((a0, records0, weight0, bias0, rows_dev0), (a1, records1, weight1, bias1, rows_dev1)):
+        _check_like(a, weight=w, bias=b, ln_weight=ln_weight, ln_bias=ln_bias)
+        if not fits_linear_layernorm(a, w):
+            raise ValueError("linear_layernorm_pair: no kernel for these operands (see fits_linear_layernorm)")
+        K = a.shape[-1]
+        a2 = a.reshape(-1, K)
+        rows = a2.shape[0]
+        if rec.shape != (rows, 16) or rec.dtype != torch.bfloat16 or not rec.is_contiguous():
+            raise ValueError(f"records must be a contiguous bfloat16 tensor of shape ({rows}, 16)")
+        wf, colrec, packed = folded_weight(w, b, ln_weight, ln_bias)
+        N = w.shape[0]
+        out = torch.empty(a.shape[:-1] + (N,), dtype=a.dtype, device=a.device)
+        outs.append(out)
+        args += [ptr(a2), a2.stride(0), ptr(rec), ptr(wf), ptr(packed), ptr(colrec), ptr(out), N, ptr(rd), rows, N]
+        shapes += (rows, N, rd is not None)
+    call("vtdge_linear_layernorm_pair", *args, a0.shape[-1], dtype_code(a0), stream_ptr(),
+         tag=("linear_layernorm_pair",) + shapes)
+    return outs[0], outs[1]
+
+
 def sparse_attention(q, k, v, offsets, scale, num_heads, max_rows_per_sample, out=None):
     """Strided form.  q [L, h*d]; k, v [B, n, h*d]-like views (last dim contiguous, any batch/token strides);
     offsets int64 [B+1] on the device.  Returns [L, h*d] with channel = head*d + j."""
