@@ -146,6 +146,21 @@ int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_
                             float records_eps, const int64_t *next_splits, uint8_t *next_counts, int B, int H, int W,
                             int C, int extra, int R, int S, int S2, int dtype, void *stream);
 
+/* The router of a model's FIRST block together with the statistics records of all its tokens (no scatter-back
+ * precedes it that could leave them): vtdge_router and vtdge_layernorm_stats in one pass over x, i.e.
+ * DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75) and the statistics half of norm1
+ * (vtpack/models/dge/deit_dge.py:127).  gate / indices are bit-identical to vtdge_router's; the records are one-pass
+ * fp32 sums about a value of the row itself, as vtdge_decompress_router writes them.
+ *   x [B, extra + H*W, C]   records [B * (extra + H*W), 16] bf16   counts (nullable) as in vtdge_decompress_router,
+ *   from `splits` int64 [S] on the device
+ *   front_rows (nullable) [extra, C]: rows that are first stored as tokens 0 .. extra-1 of EVERY sample of x - the
+ *   class (and distillation) token plus its position embedding, which the reference concatenates in front of the
+ *   patch tokens (deit_dge.py:270-277) and which do not depend on the sample.
+ * bf16 rows of 264 to 512 channels, R = 4. */
+int vtdge_router_stats(void *x, const void *front_rows, const void *weight, const void *bias, void *gate,
+                       int64_t *indices, void *records, float records_eps, const int64_t *splits, uint8_t *counts,
+                       int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream);
+
 /* Gate indices -> packed queries in one step, by region: vtdge_index_to_patch and vtdge_compress together, i.e.
  * grained_sample_index_to_patch followed by grained_sample_compress
  * (vtpack/layers/csrc/grained_sample/grained_sample.cu:302-345 with :146-196, and :198-239 with :31-69) as

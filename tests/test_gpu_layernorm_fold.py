@@ -312,6 +312,37 @@ def test_scatter_back_writes_records_of_the_tokens(dev, B, H, Cc, extra):
     assert float(((s2.double() - s_ref2) / s_ref2).abs().max()) < 3e-5
 
 
+@pytest.mark.parametrize("B,H,Cc,extra,with_front", [(8, 16, 384, 1, True), (4, 32, 384, 2, True), (3, 8, 512, 0, False),
+                                                    (2, 8, 264, 1, False)])
+def test_router_with_records_of_all_tokens(dev, B, H, Cc, extra, with_front):
+    """The first block's kernel: gate logits and indices bit for bit those of the router, the records of every token
+    row, the query counts per region, and the rows given for the extra tokens stored in every sample."""
+    from vtpack_amd import ops
+    W = H
+    N = extra + H * W
+    g = torch.Generator().manual_seed(B + Cc)
+    x = (torch.randn(B, N, Cc, generator=g) * 2 + 5 * torch.randn(B, N, 1, generator=g)).bfloat16().to(dev)
+    wgt = (torch.randn(3, Cc, generator=g) * 0.1).bfloat16().to(dev)
+    bias = (torch.randn(3, generator=g) * 0.1).bfloat16().to(dev)
+    splits = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    front = (torch.randn(extra, Cc, generator=g) * 3).bfloat16().to(dev) if with_front else None
+    want_x = x.clone()
+    if with_front:
+        want_x[:, :extra] = front
+    want_gate, want_idx = ops.router(want_x, wgt, bias, H, W, 4)
+    gate, idx, rec, counts = ops.router_stats(x, wgt, bias, H, W, 4, EPS, front_rows=front, splits=splits)
+    assert torch.equal(x, want_x)                       # only the extra-token rows were written
+    assert torch.equal(gate, want_gate) and torch.equal(idx, want_idx)
+    assert torch.equal(counts[:idx.numel()].long(), splits[idx.reshape(-1)] ** 2)
+    mean, sigma, _ = decode(rec)
+    m_ref, s_ref = want_stats(want_x)
+    assert_record_layout(rec)
+    assert float((mean.double() - m_ref).abs().max()) < 5e-6 * float(want_x.double().abs().max())
+    assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
+    _, _, rec2, none = ops.router_stats(x, wgt, bias, H, W, 4, EPS)
+    assert none is None and torch.equal(rec2, rec)
+
+
 def test_scatter_records_refused_for_other_rows(dev):
     from vtpack_amd import ops
     from vtpack_amd._lib import VtdgeError
@@ -329,8 +360,8 @@ def test_scatter_records_refused_for_other_rows(dev):
 # ----------------------------------------------------------------------------- the model with and without
 def test_model_with_and_without_folded_norms(dev):
     """DeiT-S+DGE, bf16, 256 px, batch 16 (enough rows for the weight-stationary kernels): with the folding on the
-    forward launches one statistics kernel (the first block's tokens) and one LayerNorm (the final one) instead of 25
-    LayerNorms.  Rounding differs between the two forms, so a near-tie of some router may fall the other way and the
+    forward launches one LayerNorm (the final one) instead of 37, the statistics of the first block's tokens coming
+    from its router's kernel.  Rounding differs between the two forms, so a near-tie of some router may fall the other way and the
     two runs need not route alike after the first block: each run is therefore compared with the CPU restatement
     under its OWN gate choices (logits within the bf16 bar, integer outputs of every layer exact)."""
     from vtpack_amd import _lib, engine
@@ -363,7 +394,8 @@ def test_model_with_and_without_folded_norms(dev):
         _lib.timer = None
     (on, len_on, names_on), (off, len_off, names_off) = runs[True], runs[False]
     assert names_off.count("vtdge_layernorm") == 37 and names_off.count("vtdge_linear_layernorm") == 0
-    assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 1
+    assert names_on.count("vtdge_layernorm") == 1 and names_on.count("vtdge_layernorm_stats") == 0
+    assert names_on.count("vtdge_router_stats") == 1 and names_on.count("vtdge_router") == 0
     assert names_on.count("vtdge_linear_layernorm") == 12 and names_on.count("vtdge_linear_layernorm_pair") == 12
     assert names_on.count("vtdge_linear_stats") == 12
     assert torch.equal(len_on[0], len_off[0])

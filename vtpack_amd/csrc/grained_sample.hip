@@ -900,7 +900,50 @@ __device__ __forceinline__ void region_scatter(const T *__restrict__ in, const T
     }
 }
 
-template <typename T, int GS, bool SUB, bool STAT = false>
+// The same pass over a region without the scatter (SCATTER = false below): the tokens are read, summed for the
+// router and, with STAT, their records written; nothing is stored to the tokens.
+template <typename T, bool STAT>
+__device__ __forceinline__ void region_read(const T *__restrict__ refp, int W, int C, float (&acc)[Elem<T>::VEC],
+                                            bool act, u32x4 *__restrict__ rec, float eps)
+{
+    constexpr int VEC = Elem<T>::VEC;
+#pragma unroll 1
+    for (int dy = 0; dy < 4; dy++) {
+        float pivot[4], st[8];
+        u32x4 xr[4];
+#pragma unroll
+        for (int dx = 0; dx < 4; dx++) {
+            xr[dx] = u32x4{0u, 0u, 0u, 0u};
+            if (act) xr[dx] = *reinterpret_cast<const u32x4 *>(refp + ((int64_t)dy * W + dx) * C);
+        }
+#pragma unroll
+        for (int dx = 0; dx < 4; dx++) {
+            float f[VEC];
+            Elem<T>::unpack(xr[dx], f);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) acc[c] += f[c];
+            if constexpr (STAT) {
+                pivot[dx] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(f[0])));
+                float a = 0.f, q = 0.f;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    const float d = f[c] - pivot[dx];
+                    a += d;
+                    q += d * d;
+                }
+                st[2 * dx] = act ? a : 0.f;
+                st[2 * dx + 1] = act ? q : 0.f;
+            }
+        }
+        if constexpr (STAT) write_records4(st, pivot[0], pivot[1], pivot[2], pivot[3], C, eps, rec + (int64_t)dy * W * 2);
+    }
+}
+
+// SCATTER = false: no packed rows at all - the kernel routes on `ref` as it stands and writes the records of its
+// rows (the first block of a model, which no scatter-back precedes); `in` then points, if anywhere, at `extra`
+// rows [extra, C] that are first copied into the extra-token rows of every sample of `out` (class / distillation
+// token plus their position embedding, the same for every sample).
+template <typename T, int GS, bool SUB, bool STAT = false, bool SCATTER = true>
 __global__ __launch_bounds__(256) void decompress_route_kernel(
     const T *__restrict__ in, const T *__restrict__ sub, const int64_t *__restrict__ cur_indices,
     const int64_t *__restrict__ splits, const int64_t *__restrict__ offsets, const T *__restrict__ ref,
@@ -928,15 +971,19 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
         return (int)splits[g];
     };
     // first packed row of this region (query counts are small integers: exact in fp32)
-    float before = 0.f;
-    for (int r2 = lane; r2 < rr; r2 += GS) {
-        const int ps2 = split_of((int64_t)b * nreg + r2);
-        before += (float)(ps2 * ps2);
+    int64_t row_b = 0, r0 = 0;
+    int ps = 1;
+    if constexpr (SCATTER) {
+        float before = 0.f;
+        for (int r2 = lane; r2 < rr; r2 += GS) {
+            const int ps2 = split_of((int64_t)b * nreg + r2);
+            before += (float)(ps2 * ps2);
+        }
+        row_b = offsets[b];
+        r0 = row_b + extra + (int64_t)group_sum<GS>(before);
+        ps = split_of(region);
+        if constexpr (GS == WAVE) ps = __builtin_amdgcn_readfirstlane(ps);      // one region per wave: a scalar branch
     }
-    const int64_t row_b = offsets[b];
-    const int64_t r0 = row_b + extra + (int64_t)group_sum<GS>(before);
-    int ps = split_of(region);
-    if constexpr (GS == WAVE) ps = __builtin_amdgcn_readfirstlane(ps);      // one region per wave: a scalar branch
 
     float part[VTDGE_MAX_SPLITS];
 #pragma unroll
@@ -955,7 +1002,8 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
         const T *inv = in + v * VEC;
         const T *subv = SUB ? sub + v * VEC : nullptr;
         u32x4 *rec = STAT ? records + ((int64_t)b * N + tok0) * 2 : nullptr;
-        if (ps == 4) region_scatter<T, 4, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
+        if constexpr (!SCATTER) region_read<T, STAT>(ref + off, W, C, acc, act, rec, eps);
+        else if (ps == 4) region_scatter<T, 4, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
         else if (ps == 2) region_scatter<T, 2, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
         else region_scatter<T, 1, SUB, STAT>(inv, subv, r0, ref + off, out + off, W, C, acc, act, rec, eps);
         if (rr == 0) {          // the sample's extra tokens: packed rows row_b .. row_b + extra - 1
@@ -964,21 +1012,32 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
 #pragma unroll
                 for (int c = 0; c < VEC; c++) d[c] = r[c] = 0.f;
                 const int64_t oe = ((int64_t)b * N + e) * C + v * VEC;
-                if (act) {
-                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(inv + (row_b + e) * (int64_t)C), d);
-                    if constexpr (SUB) {
-                        float sv[VEC];
-                        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(subv + (row_b + e) * (int64_t)C), sv);
+                u32x4 packed = {0u, 0u, 0u, 0u};
+                if constexpr (SCATTER) {
+                    if (act) {
+                        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(inv + (row_b + e) * (int64_t)C), d);
+                        if constexpr (SUB) {
+                            float sv[VEC];
+                            Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(subv + (row_b + e) * (int64_t)C), sv);
 #pragma unroll
-                        for (int c = 0; c < VEC; c++) d[c] -= sv[c];
-                        Elem<T>::unpack(Elem<T>::pack(d), d);      // rounded to the storage type
+                            for (int c = 0; c < VEC; c++) d[c] -= sv[c];
+                            Elem<T>::unpack(Elem<T>::pack(d), d);      // rounded to the storage type
+                        }
+                        Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + oe), r);
                     }
-                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(ref + oe), r);
-                }
 #pragma unroll
-                for (int c = 0; c < VEC; c++) r[c] += d[c];
-                const u32x4 packed = Elem<T>::pack(r);
-                if (act) *reinterpret_cast<u32x4 *>(out + oe) = packed;
+                    for (int c = 0; c < VEC; c++) r[c] += d[c];
+                    packed = Elem<T>::pack(r);
+                    if (act) *reinterpret_cast<u32x4 *>(out + oe) = packed;
+                } else if (act) {
+                    // the row as it stands, or the row given for every sample, which is put in place first
+                    if (in != nullptr) {
+                        packed = *reinterpret_cast<const u32x4 *>(inv + (int64_t)e * C);
+                        *reinterpret_cast<u32x4 *>(out + oe) = packed;
+                    } else {
+                        packed = *reinterpret_cast<const u32x4 *>(ref + oe);
+                    }
+                }
                 if constexpr (STAT) {
                     float f[VEC], st[2] = {0.f, 0.f};
                     Elem<T>::unpack(packed, f);
@@ -1468,6 +1527,32 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
 #undef VT_LAUNCH
 #undef VT_LAUNCH2
     return check_launch("decompress_router");
+}
+
+extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *weight, const void *bias, void *gate,
+                                  int64_t *indices, void *records, float records_eps, const int64_t *splits,
+                                  uint8_t *counts, int B, int H, int W, int C, int extra, int R, int S, int dtype,
+                                  void *stream)
+{
+    VT_REQUIRE(x && weight && bias && indices && records, VTDGE_ERR_ARG, "router_stats: NULL operand");
+    VT_REQUIRE(counts == nullptr || splits != nullptr, VTDGE_ERR_ARG, "router_stats: the query counts need the splits");
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && extra >= 0, VTDGE_ERR_ARG, "router_stats: bad sizes");
+    VT_REQUIRE(R == 4, VTDGE_ERR_UNSUPPORTED, "router_stats: region size %d (4 only)", R);
+    VT_REQUIRE(H % R == 0 && W % R == 0, VTDGE_ERR_ARG, "router_stats: H=%d, W=%d not multiples of region %d", H, W, R);
+    VT_REQUIRE(S >= 1 && S <= VTDGE_MAX_SPLITS, VTDGE_ERR_UNSUPPORTED, "router_stats: S=%d outside [1,%d]", S,
+               VTDGE_MAX_SPLITS);
+    if (int rc = check_channels(C, dtype, "router_stats")) return rc;
+    VT_REQUIRE(dtype == VTDGE_BF16 && group_size(C / 8) == WAVE && C / 8 <= WAVE, VTDGE_ERR_UNSUPPORTED,
+               "router_stats: statistics records are written for bf16 rows of 264 to 512 channels (C=%d)", C);
+    VT_REQUIRE(aligned16(x) && aligned16(front_rows) && aligned16(weight) && aligned16(records), VTDGE_ERR_ARG,
+               "router_stats: operands must be 16-byte aligned");
+    const int64_t regions = (int64_t)B * (H / R) * (W / R);
+    dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
+    decompress_route_kernel<bf16_t, WAVE, false, true, false><<<grid, block, 0, (hipStream_t)stream>>>(
+        (const bf16_t *)front_rows, nullptr, nullptr, splits, nullptr, (const bf16_t *)x, (bf16_t *)x,
+        (const bf16_t *)weight, (const bf16_t *)bias, (bf16_t *)gate, indices, B, H, W, C, extra, S, S,
+        (u32x4 *)records, records_eps, splits, counts);
+    return check_launch("router_stats");
 }
 
 extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,

@@ -65,6 +65,10 @@ Q_BEFORE_KV = True
 # (`vtdge_linear_layernorm_pair`): alone the q Linear has three or four tiles per workgroup behind the fixed cost of
 # fetching its weights.
 PAIR_KV_Q = True
+# The first block of a model has no scatter-back before it to route it and to leave the statistics of its tokens:
+# one kernel does both (`vtdge_router_stats`) instead of a router and a statistics pass, and stores the class-token
+# rows on the way.
+ROUTER_STATS = True
 
 
 def _side_stream(device, slot=0):
@@ -81,6 +85,8 @@ def prepare(model):
     (`p.data.copy_(...)`, `p.data.mul_(...)`) and, optionally, before capturing a graph so that no packing kernel lands
     in the capture."""
     ops.invalidate_packed(model)
+    if getattr(model, "_vtdge_front", None) is not None:
+        object.__setattr__(model, "_vtdge_front", None)
     for mod in model.modules():
         if hasattr(mod, "_vtdge_khwc"):
             mod._vtdge_khwc = None
@@ -168,6 +174,18 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
     main = torch.cuda.current_stream(x.device)
     side = _side_stream(x.device, main.cuda_stream) if overlap else main
     swap = overlap and ROUTING_ON_SIDE
+
+    front = carry.get("front")
+    if (ROUTER_STATS and routed is None and gate is None and x_ln is None and fold1 and R == 4
+            and not FUSE_ROUTER_NORM and ops.fits_scatter_stats(x)):
+        # a model's first block: its router, the statistics records of all tokens for norm1 -> kv, the query counts
+        # of its regions and, on the way, the class-token rows put in front of every sample, in one pass over x
+        g0, i0, rec0, cnt0 = ops.router_stats(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R, n1.eps,
+                                              front_rows=front, splits=dge.splits if use_regions else None)
+        routed = (g0, i0)
+        carry = dict(carry, x_stats=rec0, counts=cnt0)
+    elif front is not None:
+        x[:, :front.shape[0], :] = front
 
     fuse_rn = (FUSE_ROUTER_NORM and gate is None and routed is None and x_ln is None
                and ops.fits_router_layernorm(x, R))
@@ -317,15 +335,31 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
     return out
 
 
-def _run_blocks(blocks, x, H, W):
-    """A chain of blocks on one token grid, each handing the next what it has already computed for it."""
-    carry = None
+def _run_blocks(blocks, x, H, W, front=None):
+    """A chain of blocks on one token grid, each handing the next what it has already computed for it.  `front`
+    [extra, C]: rows the first block stores as the extra tokens of every sample before anything reads them."""
+    carry = {"front": front} if front is not None else None
     for i, blk in enumerate(blocks):
         if i + 1 < len(blocks):
             x, carry = block_forward(blk, x, H, W, carry=carry, next_block=blocks[i + 1])
         else:
             x = block_forward(blk, x, H, W, carry=carry)
     return x
+
+
+def _front_rows(model, front):
+    """[extra, C]: the class (and distillation) token plus its row of the position table - what the reference puts
+    in front of every sample's patch tokens (deit_dge.py:270-277).  The same for every sample and every call: made
+    once per set of parameter versions and kept on the model."""
+    parts = front + [model.pos_embed]
+    key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in parts)
+    cached = getattr(model, "_vtdge_front", None)
+    if cached is None or cached[0] != key:
+        with torch.no_grad():
+            rows = (torch.cat([t.detach() for t in front], dim=1) + model.pos_embed.detach()[:, :len(front), :])[0]
+        cached = (key, rows.contiguous())
+        object.__setattr__(model, "_vtdge_front", cached)
+    return cached[1]
 
 
 def model_forward(model, images):
@@ -350,9 +384,9 @@ def model_forward(model, images):
     if FUSE_PATCH_EMBED and ops.fits_patch_embed(images, pe.proj.weight, pe.proj.bias, model.pos_embed, P):
         # the convolution reads the images in place and adds the position embedding on its way out
         x = ops.patch_embed(images, pe.proj.weight, pe.proj.bias, model.pos_embed, P, extra)
-        for e, t in enumerate(front):
-            x[:, e:e + 1, :] = t + model.pos_embed[:, e:e + 1, :]
+        front_rows = _front_rows(model, front) if extra else None
     else:
+        front_rows = None
         patches = images.reshape(B, Cin, G, P, G, P).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, Cin * P * P)
         x = torch.empty((B, extra + G * G, C), dtype=images.dtype, device=images.device)
         tok = ops.linear(patches, pe.proj.weight.reshape(C, Cin * P * P), pe.proj.bias)
@@ -360,7 +394,7 @@ def model_forward(model, images):
         for e, t in enumerate(front):
             x[:, e:e + 1, :] = t
         x += model.pos_embed
-    x = _run_blocks(list(model.blocks), x, G, G)
+    x = _run_blocks(list(model.blocks), x, G, G, front=front_rows)
     nrm = model.norm
 
     def head(lin, t):

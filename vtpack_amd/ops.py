@@ -285,6 +285,40 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
     return res
 
 
+def router_stats(x, weight, bias, H, W, region_size, stats_eps, front_rows=None, splits=None, want_gate=True):
+    """`router` and `layernorm_stats` of every token in one pass over x [B, extra + H*W, C] (bf16, see
+    `fits_scatter_stats`): -> (gate or None, indices, records [B*N, 16], counts or None).  `front_rows` [extra, C] are
+    first written into the extra-token rows of every sample of x (in place); with `splits` (int64, device) the uint8
+    query counts per region are left for `compress_regions`."""
+    _need_gpu(x, weight, bias, front_rows, splits)
+    if not x.is_contiguous():
+        raise ValueError("router_stats works on x in place: it must be contiguous")
+    B, N, C = x.shape
+    S = weight.shape[0]
+    extra = N - H * W
+    weight, bias = _contig(weight), _contig(bias)
+    _check_like(x, weight=weight, bias=bias, front_rows=front_rows)
+    _check_router(weight, bias, C, S, extra, H, W, region_size)
+    if front_rows is not None:
+        front_rows = _contig(front_rows.reshape(-1, C))
+        if front_rows.shape[0] != extra:
+            raise ValueError(f"front_rows holds {front_rows.shape[0]} rows, the tokens have {extra} in front")
+    Hr, Wr = H // region_size, W // region_size
+    gate = torch.empty((B, Hr, Wr, S), dtype=x.dtype, device=x.device) if want_gate else None
+    indices = torch.empty((B, Hr, Wr), dtype=torch.int64, device=x.device)
+    rec = torch.empty((B * N, 16), dtype=torch.bfloat16, device=x.device)
+    counts = None
+    if splits is not None:
+        if splits.dtype != torch.int64 or splits.numel() != S:
+            raise ValueError("splits must be int64 with one entry per row of the router's weight")
+        splits = _contig(splits)
+        counts = region_counts_buffer(B, Hr * Wr, x.device)
+    call("vtdge_router_stats", ptr(x), ptr(front_rows), ptr(weight), ptr(bias), ptr(gate), ptr(indices), ptr(rec),
+         float(stats_eps), ptr(splits), ptr(counts), B, H, W, C, extra, region_size, S, dtype_code(x), stream_ptr(),
+         tag=("router_stats", C))
+    return gate, indices, rec, counts
+
+
 def fits_scatter_stats(x):
     """Whether `decompress_router` can write statistics records for rows like those of x [B, N, C]."""
     return x.is_cuda and x.dtype == torch.bfloat16 and 264 <= x.shape[-1] <= 512 and x.shape[-1] % 8 == 0
