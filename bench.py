@@ -80,8 +80,7 @@ def kernel_symbol(name, tag, dt, n_keys=0):
             return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false, false>"
         return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
     if name == "vtdge_patch_embed":           # tag = ("patch_embed", B, S, patch, C)
-        big = tag[4] >= 768 or -(-(tag[1] * (tag[2] // tag[3]) ** 2) // 256) * -(-tag[4] // 128) >= 512
-        tile = "256, 128, 4, 2, 4" if big else "128, 128, 2, 2, 4"
+        tile = "256, 128, 4, 2, 4" if tag[4] >= 768 else "128, 128, 2, 2, 4"
         return f"linear_dma_kernel<{T}, {tile}, 0, true, true, 3, false, true>"
     if name == "vtdge_patch_linear":          # tag = ("patch_linear", B, H, W, C, k, N)
         rows = tag[1] * (tag[2] // tag[5]) * (tag[3] // tag[5])

@@ -416,11 +416,10 @@ int launch_patch_embed(const void *images, const void *W, const void *bias, cons
     const int G = S / P;
     const PatchGeom pg{P, S, G, Cin, extra, 0, 0, 0};
     LinArgs a{images, 0, W, bias, pos, N, out, N, nullptr, (int64_t)B * G * G, N, Cin * P * P, VTDGE_ACT_NONE, st};
-    // 256x128 tiles (half the passes over the weights, one workgroup per CU) once they give every CU two tiles and
-    // more; 128x128 tiles, two workgroups per CU, for smaller batches.  At 256 x 256 patches and N = 384: 67 against
-    // 78 us; 128x192 tiles 69 us, 128x384 tiles on a two-stage ring 93 us.
-    if (N >= 768 || ceil_div((int64_t)B * G * G, 256) * ceil_div(N, 128) >= 512)
-        return go<T, 256, 128, 4, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
+    // 128x128 tiles, two workgroups per CU, unless the output is wide.  At 256 x 256 patches and N = 384 a launch takes
+    // 80 - 88 us against 125 - 138 us on 256x128 tiles with one workgroup per CU (which only looks faster, 67 against
+    // 78 us, when launches are timed back to back and the tail of one hides under the head of the next).
+    if (N >= 768) return go<T, 256, 128, 4, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
     return go<T, 128, 128, 2, 2, 4, VTDGE_ACT_NONE, true, true, true>(a, pg);
 }
 
