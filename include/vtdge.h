@@ -139,12 +139,16 @@ int vtdge_decompress_layernorm(const void *in, const void *sub, const int64_t *p
  * vtdge_linear_layernorm; one-pass fp32 sums about a value of the row itself.  bf16 rows of 264 to 512 channels.
  * next_counts (nullable; needs the next router) uint8 [B * H/R * W/R]: the number of queries the next block takes
  * from every region, next_splits[next_indices]^2 with next_splits int64 [S2] on the device: what
- * vtdge_compress_regions adds up to place a region's queries. */
+ * vtdge_compress_regions adds up to place a region's queries.
+ * region_rows (nullable) int32 [B * H/R * W/R] with cur_counts uint8 of the same length: the first packed row and the
+ * query count of every region of THIS block as vtdge_compress_regions left them; the kernel then takes a region's
+ * place from them instead of adding it up from cur_indices and offsets. */
 int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits,
                             const int64_t *offsets, const void *ref, void *out, const void *next_weight,
                             const void *next_bias, void *next_gate, int64_t *next_indices, void *out_records,
-                            float records_eps, const int64_t *next_splits, uint8_t *next_counts, int B, int H, int W,
-                            int C, int extra, int R, int S, int S2, int dtype, void *stream);
+                            float records_eps, const int64_t *next_splits, uint8_t *next_counts,
+                            const int32_t *region_rows, const uint8_t *cur_counts, int B, int H, int W, int C,
+                            int extra, int R, int S, int S2, int dtype, void *stream);
 
 /* The router of a model's FIRST block together with the statistics records of all its tokens (no scatter-back
  * precedes it that could leave them): vtdge_router and vtdge_layernorm_stats in one pass over x, i.e.
@@ -174,13 +178,14 @@ int vtdge_router_stats(void *x, const void *front_rows, const void *weight, cons
  *           sqrt(var + records_eps), see vtdge_layernorm_stats) for a vtdge_linear_layernorm that takes comp next
  *           (norm1 -> q, vtpack/models/dge/deit_dge.py:127 with :72); bf16 only
  *   patches (nullable), offsets [B+1], lengths [B]: as vtdge_index_to_patch writes them
+ *   region_rows (nullable) int32 [B * H/R * W/R]: the first packed row of every region, for vtdge_decompress_router
  * The caller guarantees capacity_rows >= the number of queries (B * (extra + H*W) always is).  R must be 4 with splits
  * out of {1, 2, 4}, a row one 16-byte vector per lane (C <= 512 in bf16, 256 in fp32), at most 65536 regions and
  * 64 extra tokens; VTDGE_ERR_UNSUPPORTED otherwise. */
 int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t *splits, const uint8_t *counts,
                            void *comp, void *records, float records_eps, int64_t *patches, int64_t capacity_rows,
-                           int64_t *offsets, int64_t *lengths, int B, int H, int W, int C, int extra, int R, int S,
-                           int dtype, void *stream);
+                           int64_t *offsets, int64_t *lengths, int32_t *region_rows, int B, int H, int W, int C,
+                           int extra, int R, int S, int dtype, void *stream);
 
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */

@@ -756,6 +756,17 @@ def test_scatter_back_with_the_next_router(dev, dtype, B, Hr, Wr, C, extra):
                                                     next_bias=bias, next_splits=splits)
     assert torch.equal(nidx, want_idx) and counts.dtype == torch.uint8
     assert torch.equal(counts[:nidx.numel()].long(), (splits[nidx.reshape(-1)] ** 2))
+    # a region's place handed over by compress_regions instead of added up from the gate indices
+    cur = ops.region_counts_buffer(B, (H // 4) * (W // 4), dev)
+    cur[:idx.numel()] = (splits[idx.reshape(-1)] ** 2).to(torch.uint8)
+    per = (splits[idx.reshape(B, -1)] ** 2)
+    rrows = (offsets[:B, None] + extra + per.cumsum(1) - per).reshape(-1).to(torch.int32)
+    if ops.fits_compress_regions(x, H, W, 4, SPLITS):           # and that is what compress_regions leaves
+        assert torch.equal(ops.compress_regions(x, idx, splits, H, W, 4, counts=cur, want_region_rows=True)[5], rrows)
+    placed = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp, next_weight=wgt, next_bias=bias,
+                                   region_rows=rrows, cur_counts=cur)
+    want = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp, next_weight=wgt, next_bias=bias)
+    assert all(torch.equal(a, b) for a, b in zip(placed, want))
     # without a next router it is the plain scatter-back
     alone, g0, i0 = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=comp)
     assert g0 is None and i0 is None

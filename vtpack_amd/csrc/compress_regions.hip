@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void compress_regions_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ indices, const int64_t *__restrict__ splits,
     const uint8_t *__restrict__ counts, T *__restrict__ comp, u32x4 *__restrict__ records,
     int64_t *__restrict__ patches, int64_t capacity, int64_t *__restrict__ offsets, int64_t *__restrict__ lengths,
-    int B, int H, int W, int C, int extra, int S, float eps)
+    int32_t *__restrict__ region_rows, int B, int H, int W, int C, int extra, int S, float eps)
 {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int R = 4;
@@ -89,10 +89,18 @@ __global__ __launch_bounds__(256) void compress_regions_kernel(
         for (int i = lane; i < region; i += WAVE) before += (float)count_of(i);
     }
     const int64_t r0 = (int64_t)wave_sum(before) + (int64_t)extra * (b + 1);      // first packed row of the region
-    int64_t gi = indices[region];
-    gi = gi < 0 ? 0 : (gi >= S ? S - 1 : gi);
-    const int ps = __builtin_amdgcn_readfirstlane((int)splits[gi]);
+    // the region's own split: from its count byte when there is one (no trip through the indices and the splits)
+    int ps;
+    if (counts != nullptr) {
+        const int cnt = __builtin_amdgcn_readfirstlane((int)counts[region]);
+        ps = cnt == 16 ? 4 : cnt == 4 ? 2 : 1;
+    } else {
+        int64_t gi = indices[region];
+        gi = gi < 0 ? 0 : (gi >= S ? S - 1 : gi);
+        ps = __builtin_amdgcn_readfirstlane((int)splits[gi]);
+    }
     const int nq = ps == 4 ? 16 : ps == 2 ? 4 : 1;
+    if (region_rows != nullptr && lane == 0) region_rows[region] = (int32_t)r0;
 
     // ---- the bookkeeping index->patch leaves: descriptors, offsets, lengths
     if (patches != nullptr && lane < nq) {
@@ -240,7 +248,8 @@ using namespace vtdge;
 extern "C" int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t *splits,
                                       const uint8_t *counts, void *comp, void *records, float records_eps,
                                       int64_t *patches, int64_t capacity_rows, int64_t *offsets, int64_t *lengths,
-                                      int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream)
+                                      int32_t *region_rows, int B, int H, int W, int C, int extra, int R, int S,
+                                      int dtype, void *stream)
 {
     VT_REQUIRE(x && indices && splits && comp && offsets && lengths, VTDGE_ERR_ARG, "compress_regions: NULL operand");
     VT_REQUIRE(B > 0 && H > 0 && W > 0 && extra >= 0 && capacity_rows >= 0, VTDGE_ERR_ARG, "compress_regions: bad sizes");
@@ -267,7 +276,7 @@ extern "C" int vtdge_compress_regions(const void *x, const int64_t *indices, con
 #define VT_LAUNCH(T, RECF)                                                                                         \
     compress_regions_kernel<T, RECF><<<grid, block, 0, st>>>((const T *)x, indices, splits, counts, (T *)comp,     \
                                                              (u32x4 *)records, patches, capacity_rows, offsets,    \
-                                                             lengths, B, H, W, C, extra, S, records_eps)
+                                                             lengths, region_rows, B, H, W, C, extra, S, records_eps)
     if (dtype == VTDGE_F32) VT_LAUNCH(float, false);
     else if (records != nullptr) VT_LAUNCH(bf16_t, true);
     else VT_LAUNCH(bf16_t, false);

@@ -950,7 +950,8 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
     T *__restrict__ out, const T *__restrict__ weight, const T *__restrict__ bias, T *__restrict__ gate,
     int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2,
     u32x4 *__restrict__ records = nullptr, float eps = 0.f, const int64_t *__restrict__ next_splits = nullptr,
-    uint8_t *__restrict__ next_counts = nullptr)
+    uint8_t *__restrict__ next_counts = nullptr, const int32_t *__restrict__ region_rows = nullptr,
+    const uint8_t *__restrict__ cur_counts = nullptr)
 {
     static_assert(!STAT || (GS == WAVE && std::is_same<T, bf16_t>::value), "records: one wave per region, bf16 rows");
     constexpr int VEC = Elem<T>::VEC;
@@ -974,14 +975,22 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
     int64_t row_b = 0, r0 = 0;
     int ps = 1;
     if constexpr (SCATTER) {
-        float before = 0.f;
-        for (int r2 = lane; r2 < rr; r2 += GS) {
-            const int ps2 = split_of((int64_t)b * nreg + r2);
-            before += (float)(ps2 * ps2);
+        if (region_rows != nullptr) {
+            // the kernel that packed the rows has left every region's first row and query count: one load each
+            r0 = region_rows[region];
+            row_b = r0 - extra;          // read for a sample's first region only
+            const int cnt = cur_counts[region];
+            ps = cnt == 16 ? 4 : cnt == 4 ? 2 : 1;
+        } else {
+            float before = 0.f;
+            for (int r2 = lane; r2 < rr; r2 += GS) {
+                const int ps2 = split_of((int64_t)b * nreg + r2);
+                before += (float)(ps2 * ps2);
+            }
+            row_b = offsets[b];
+            r0 = row_b + extra + (int64_t)group_sum<GS>(before);
+            ps = split_of(region);
         }
-        row_b = offsets[b];
-        r0 = row_b + extra + (int64_t)group_sum<GS>(before);
-        ps = split_of(region);
         if constexpr (GS == WAVE) ps = __builtin_amdgcn_readfirstlane(ps);      // one region per wave: a scalar branch
     }
 
@@ -1479,9 +1488,12 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
                                        const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
                                        const void *next_weight, const void *next_bias, void *next_gate,
                                        int64_t *next_indices, void *out_records, float records_eps,
-                                       const int64_t *next_splits, uint8_t *next_counts, int B, int H, int W, int C,
-                                       int extra, int R, int S, int S2, int dtype, void *stream)
+                                       const int64_t *next_splits, uint8_t *next_counts, const int32_t *region_rows,
+                                       const uint8_t *cur_counts, int B, int H, int W, int C, int extra, int R, int S,
+                                       int S2, int dtype, void *stream)
 {
+    VT_REQUIRE((region_rows == nullptr) == (cur_counts == nullptr), VTDGE_ERR_ARG,
+               "decompress_router: the regions' first rows and their query counts come together");
     VT_REQUIRE(next_counts == nullptr || (next_splits != nullptr && next_indices != nullptr), VTDGE_ERR_ARG,
                "decompress_router: the next block's query counts need its router and its splits");
     VT_REQUIRE(in && cur_indices && splits && offsets && ref && out, VTDGE_ERR_ARG, "decompress_router: NULL operand");
@@ -1508,7 +1520,7 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
     decompress_route_kernel<bf16_t, WAVE, SUBF, true><<<grid, block, 0, st>>>(                                       \
         (const bf16_t *)in, (const bf16_t *)sub, cur_indices, splits, offsets, (const bf16_t *)ref, (bf16_t *)out,   \
         (const bf16_t *)next_weight, (const bf16_t *)next_bias, (bf16_t *)next_gate, next_indices, B, H, W, C, extra, \
-        S, S2, (u32x4 *)out_records, records_eps, next_splits, next_counts)
+        S, S2, (u32x4 *)out_records, records_eps, next_splits, next_counts, region_rows, cur_counts)
         if (sub) VT_STAT(true); else VT_STAT(false);
 #undef VT_STAT
         return check_launch("decompress_router");
@@ -1517,7 +1529,7 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
     decompress_route_kernel<T, GS, SUBF><<<grid, block, 0, st>>>(                                                  \
         (const T *)in, (const T *)sub, cur_indices, splits, offsets, (const T *)ref, (T *)out,                     \
         (const T *)next_weight, (const T *)next_bias, (T *)next_gate, next_indices, B, H, W, C, extra, S, S2,      \
-        nullptr, 0.f, next_splits, next_counts)
+        nullptr, 0.f, next_splits, next_counts, region_rows, cur_counts)
 #define VT_LAUNCH(T, GS) do { if (sub) VT_LAUNCH2(T, GS, true); else VT_LAUNCH2(T, GS, false); } while (0)
 #define VT_GROUP(T) \
     do { if (gs == 64) VT_LAUNCH(T, 64); else if (gs == 32) VT_LAUNCH(T, 32); else if (gs == 16) VT_LAUNCH(T, 16); \

@@ -69,6 +69,9 @@ PAIR_KV_Q = True
 # one kernel does both (`vtdge_router_stats`) instead of a router and a statistics pass, and stores the class-token
 # rows on the way.
 ROUTER_STATS = True
+# `vtdge_compress_regions` leaves every region's first packed row for the scatter-back of the same block, which then
+# needs no sum over the gate indices before it can start on its rows.
+REGION_ROWS = True
 
 
 def _side_stream(device, slot=0):
@@ -206,6 +209,7 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         return src, ops.linear(src, attn.kv.weight, attn.kv.bias)             # [B, n, 2C] = [B, n, 2, h, d]
 
     cap = B * N
+    placed = {}      # where compress_regions has put every region's rows, for the scatter-back of this block
 
     def routing_chain():
         """-> (gate, indices, patches, offsets, lengths, comp, LayerNorm(comp) or None, records of comp or None)"""
@@ -222,9 +226,12 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
             # index->patch and compress in one kernel, by region; with the folded norm1 -> q it leaves the statistics
             # records of the packed rows instead of their normalised copy
             foldq = FOLD_NORMS and ops.fits_linear_layernorm(x, attn.q.weight)
-            cmp_, rec, pat, off, lens = ops.compress_regions(
-                x, idx, dge.splits, H, W, R, counts=carry.get("counts") if routed is not None else None,
-                stats_eps=n1.eps if foldq else None, capacity=cap)
+            cnt = carry.get("counts") if routed is not None else None
+            cmp_, rec, pat, off, lens, rrows = ops.compress_regions(
+                x, idx, dge.splits, H, W, R, counts=cnt, stats_eps=n1.eps if foldq else None, capacity=cap,
+                want_region_rows=True)
+            if cnt is not None and REGION_ROWS:
+                placed["region_rows"], placed["cur_counts"] = rrows, cnt
             ln = None if foldq else ops.layernorm(cmp_, n1.weight, n1.bias, n1.eps, rows_dev=off[B:])
             return g, idx, pat, off, lens, cmp_, ln, rec
         pat, off, lens = ops.index_to_patch(idx, dge.splits, R, extra, capacity=cap)
@@ -308,7 +315,7 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         res = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
                                     next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias,
                                     stats_eps=next_block.norm1.eps if want_stats else None,
-                                    next_splits=nxt.splits if want_counts else None)
+                                    next_splits=nxt.splits if want_counts else None, **placed)
         out, ngate, nidx = res[:3]
         handed["routed"] = (ngate, nidx)
         if want_stats:

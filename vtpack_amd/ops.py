@@ -195,13 +195,14 @@ def fits_compress_regions(x, H, W, region_size, split_sizes):
 
 
 def compress_regions(x, indices, splits, H, W, region_size=4, counts=None, stats_eps=None, capacity=None,
-                     want_patches=True):
+                     want_patches=True, want_region_rows=False):
     """index_to_patch and compress in one kernel, by region: x [B, extra + H*W, C] and the gate indices [B, Hr, Wr]
     -> (comp [capacity, C], records or None, patches or None, offsets [B+1], lengths [B]).  `counts` is the uint8
     buffer a `decompress_router(..., next_splits=...)` has filled for these indices (optional: the kernel otherwise
     works the counts out from the indices); with `stats_eps` (bf16) the statistics records of the rows of comp are
     written for a `linear_layernorm` that takes comp next.  comp, patches, offsets and lengths equal those of
-    `index_to_patch` + `compress` bit for bit.  vtpack/layers/dge.py:76-79."""
+    `index_to_patch` + `compress` bit for bit.  With `want_region_rows` a sixth value: int32 [B * regions], the first
+    packed row of every region (for the `decompress_router` of the same block).  vtpack/layers/dge.py:76-79."""
     _need_gpu(x, indices, splits, counts)
     x, indices, splits = _contig(x), _contig(indices), _contig(splits)
     if indices.dtype != torch.int64 or splits.dtype != torch.int64 or indices.dim() != 3:
@@ -224,21 +225,26 @@ def compress_regions(x, indices, splits, H, W, region_size=4, counts=None, stats
     patches = torch.empty((capacity, 4), dtype=torch.int64, device=x.device) if want_patches else None
     offsets = torch.empty((B + 1,), dtype=torch.int64, device=x.device)
     lengths = torch.empty((B,), dtype=torch.int64, device=x.device)
+    region_rows = torch.empty((B * regions,), dtype=torch.int32, device=x.device) if want_region_rows else None
     call("vtdge_compress_regions", ptr(x), ptr(indices), ptr(splits), ptr(counts), ptr(comp), ptr(rec),
          float(stats_eps if stats_eps is not None else 0.0), ptr(patches), capacity, ptr(offsets), ptr(lengths),
-         B, H, W, C, extra, region_size, splits.numel(), dtype_code(x), stream_ptr(),
+         ptr(region_rows), B, H, W, C, extra, region_size, splits.numel(), dtype_code(x), stream_ptr(),
          tag=("compress_regions", rec is not None, C, counts is not None))
+    if want_region_rows:
+        return comp, rec, patches, offsets, lengths, region_rows
     return comp, rec, patches, offsets, lengths
 
 
 def decompress_router(inp, indices, splits, offsets, reference, H, W, region_size, sub=None, next_weight=None,
-                      next_bias=None, want_gate=True, stats_eps=None, next_splits=None):
+                      next_bias=None, want_gate=True, stats_eps=None, next_splits=None, region_rows=None,
+                      cur_counts=None):
     """Scatter (inp - sub) + reference back over the tokens by region, and route the NEXT block on the result:
     -> (out, next_gate or None, next_indices or None), and with `stats_eps` (a LayerNorm's eps; bf16 rows of 264 to
     512 channels) a fourth value: the statistics records of the rows of `out` for `linear_layernorm`; with `next_splits`
     (the next block's split sizes, int64 on the device) one more at the end: the uint8 query counts of the next block's
     regions for `compress_regions`.  `indices` [B, Hr, Wr] are this block's gate indices, `offsets` [B+1] the prefix of
-    its query counts.  The three outputs equal decompress(...) and router(out, next_weight,
+    its query counts; `region_rows` with `cur_counts` (from this block's `compress_regions` and the count bytes it
+    read) spare the kernel adding a region's place up from them.  The three outputs equal decompress(...) and router(out, next_weight,
     next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75."""
     _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
     inp, reference = _contig(inp), _contig(reference)
@@ -275,11 +281,20 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
             raise ValueError("next_splits goes with the next router: int64, one entry per row of next_weight")
         _need_gpu(next_splits)
         next_splits = _contig(next_splits)
+    if (region_rows is None) != (cur_counts is None):
+        raise ValueError("region_rows (from compress_regions) and cur_counts (this block's count bytes) go together")
+    if region_rows is not None:
+        _need_gpu(region_rows, cur_counts)
+        nr = B * (H // region_size) * (W // region_size)
+        if region_rows.dtype != torch.int32 or region_rows.numel() != nr or cur_counts.dtype != torch.uint8 \
+                or cur_counts.numel() < nr:
+            raise ValueError("region_rows must be int32 with one entry per region, cur_counts the uint8 buffer beside it")
+    if next_splits is not None:
         counts = region_counts_buffer(B, (H // region_size) * (W // region_size), inp.device)
     call("vtdge_decompress_router", ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference),
          ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), ptr(rec),
-         float(stats_eps if stats_eps is not None else 0.0), ptr(next_splits), ptr(counts), B, H, W, C, extra,
-         region_size, S, S2, dtype_code(inp), stream_ptr(),
+         float(stats_eps if stats_eps is not None else 0.0), ptr(next_splits), ptr(counts), ptr(region_rows),
+         ptr(cur_counts), B, H, W, C, extra, region_size, S, S2, dtype_code(inp), stream_ptr(),
          tag=("decompress_router", sub is not None, next_weight is not None, C, rec is not None))
     res = (out, gate, nidx) + ((rec,) if stats_eps is not None else ()) + ((counts,) if counts is not None else ())
     return res
