@@ -40,8 +40,9 @@ WORKLOADS = {
 class EventTimer:
     """Brackets every libvtdge call with a pair of HIP events on the stream the kernels are launched on."""
 
-    def __init__(self, torch):
+    def __init__(self, torch, last_kernel):
         self.torch = torch
+        self.last_kernel = last_kernel
         self.records = []
         self._open = None
 
@@ -54,75 +55,13 @@ class EventTimer:
     def end(self):
         name, tag, s, e = self._open
         e.record()
-        self.records.append((name, tag, s, e))
+        # the kernel the call has just launched, under the name the library itself reports for it (the one
+        # rocprofv3 lists): the per-kernel table below cannot drift from the library's dispatch
+        self.records.append((name, tag, s, e, self.last_kernel()))
 
     def durations(self):
         self.torch.cuda.synchronize()
-        return [(n, t, s.elapsed_time(e) * 1e-3) for n, t, s, e in self.records]
-
-
-def kernel_symbol(name, tag, dt, n_keys=0):
-    """Name under which rocprofv3 lists the kernel a call launches (T = float or unsigned short).
-
-    Mirrors the host-side dispatch of libvtdge for the shapes of these workloads (all operands 16-byte aligned)."""
-    T = "unsigned short" if dt == "bf16" else "float"
-    esz = 2 if dt == "bf16" else 4
-    b = lambda v: "true" if v else "false"  # noqa: E731
-    if name in ("vtdge_linear", "vtdge_linear_prepacked"):
-        act = 1 if tag[1] == "gelu" else 0
-        rows, N, K = tag[4], tag[5], tag[6]
-        if dt == "bf16" and K == 384 and N % 384 == 0 and N // 384 <= 8 and rows >= 2048 and not (act and tag[3]):
-            return f"linear_ws8_kernel<{act}, {b(tag[2])}, {b(tag[3])}, false, false>"
-        if dt == "bf16" and K == 1536 and N % 96 == 0 and N // 96 <= 8 and rows >= 2048 and not act:
-            return f"linear_ks_kernel<{b(tag[2])}, {b(tag[3])}>"
-        if (K * esz) % 128 == 0 and N % (16 // esz) == 0:
-            tile = "256, 128, 4, 2, 4" if N >= 768 else "128, 128, 2, 2, 4"
-            return f"linear_dma_kernel<{T}, {tile}, {act}, {b(tag[2])}, {b(tag[3])}, 3, false, false>"
-        return f"linear_kernel<{T}, {act}, {b(tag[2])}, {b(tag[3])}>"
-    if name == "vtdge_patch_embed":           # tag = ("patch_embed", B, S, patch, C)
-        tile = "256, 128, 4, 2, 4" if tag[4] >= 768 else "128, 128, 2, 2, 4"
-        return f"linear_dma_kernel<{T}, {tile}, 0, true, true, 3, false, true>"
-    if name == "vtdge_patch_linear":          # tag = ("patch_linear", B, H, W, C, k, N)
-        rows = tag[1] * (tag[2] // tag[5]) * (tag[3] // tag[5])
-        big = tag[6] >= 768 or -(-rows // 256) * -(-tag[6] // 128) >= 512
-        tile = "256, 128, 4, 2, 4" if big else "128, 128, 2, 2, 4"
-        return f"linear_dma_kernel<{T}, {tile}, 0, true, false, 3, false, true>"
-    if name == "vtdge_linear_layernorm":
-        return f"linear_ws8_kernel<{1 if tag[1] == 'gelu' else 0}, false, false, true, false>"
-    if name == "vtdge_linear_layernorm_pair":
-        return "linear_ws8_pair_kernel<0>"
-    if name == "vtdge_linear_stats":
-        return f"linear_ws8_kernel<0, {b(tag[1])}, {b(tag[2])}, false, true>"
-    if name == "vtdge_compress_regions":
-        return f"compress_regions_kernel<{T}, {b(tag[1])}>"
-    gs = lambda C: (lambda nv: 64 if nv > 32 else 32 if nv > 16 else 16 if nv > 8 else 8)(C * esz // 16)  # noqa: E731
-    if name == "vtdge_layernorm_stats":
-        nv = tag[2] * esz // 16
-        return f"layernorm_stats_kernel<{min(3, -(-nv // 64)) if gs(tag[2]) == 64 else 1}, {gs(tag[2])}>"
-    if name == "vtdge_compress":
-        return f"compress_kernel<{T}, {b(tag[1])}, {gs(tag[3])}, {3 if tag[3] * esz // 16 > 64 else 1}>"
-    if name == "vtdge_decompress":
-        return f"decompress_kernel<{T}, {b(tag[1])}, {b(tag[2])}, {gs(tag[3])}>"
-    if name == "vtdge_decompress_layernorm":
-        return f"decompress_ln_kernel<{T}, {b(tag[1])}, {gs(tag[2])}>"
-    if name == "vtdge_decompress_router":
-        return f"decompress_route_kernel<{T}, {gs(tag[3])}, {b(tag[1])}, {b(tag[4])}>"
-    if name == "vtdge_layernorm":
-        nv = tag[3] * esz // 16                           # 16-byte vectors per row
-        return f"layernorm_kernel<{T}, {min(3, -(-nv // 64)) if gs(tag[3]) == 64 else 1}, {gs(tag[3])}>"
-    if name == "vtdge_sparse_attention":
-        if dt == "bf16" and tag[3] == 64:
-            if tag[4] <= 288:
-                return f"sparse_attention_bf16_d64_pipelined_kernel<{-(-tag[4] // 32)}>"
-            return "sparse_attention_bf16_d64_stream_kernel"
-        return f"sparse_attention_kernel<{T}, {tag[3]}>"
-    if name == "vtdge_router":
-        return f"router_kernel<{T}, 4, {gs(tag[1])}, false>"     # region size 4 in every model of these workloads
-    if name == "vtdge_router_layernorm":
-        return f"router_kernel<{T}, 4, {gs(tag[1])}, true>"
-    if name == "vtdge_index_to_patch":
-        return "patch_write_kernel<true>"      # one launch for batch * regions <= 16384 (all workloads here)
-    return name
+        return [(n, t, s.elapsed_time(e) * 1e-3, k) for n, t, s, e, k in self.records]
 
 
 def measured_traffic(workload):
@@ -202,6 +141,9 @@ def algorithmic_work(name, tag, esz, geo):
         return "hbm", 2.0 * rows * tag[3] * esz
     if name == "vtdge_router":
         return "hbm", B * (N - geo["extra"]) * C * esz
+    if name == "vtdge_router_stats":
+        # every token read once, a 32-byte record written per token
+        return "hbm", B * N * C * esz + 32.0 * B * N
     if name == "vtdge_router_layernorm":
         return "hbm", 2.0 * B * N * C * esz              # every token read once, its LayerNorm written once
     if name == "vtdge_index_to_patch":
@@ -279,7 +221,7 @@ def run_model_workload(args, torch):
     value = batch * args.steps / dt_s
 
     # ---- per-kernel HIP-event timing: the same steps again, eagerly, every libvtdge launch bracketed
-    timer = EventTimer(torch)
+    timer = EventTimer(torch, _lib.last_kernel)
     inst_steps = min(args.steps, 5)
     lens = []
     _lib.timer = timer
@@ -304,13 +246,12 @@ def run_model_workload(args, torch):
     per_step = len(recs) // inst_steps
     stats = {}
     blk = 0
-    for i, (name, tag, sec) in enumerate(recs):
+    for i, (name, tag, sec, sym) in enumerate(recs):
         if i % per_step == 0:
             blk = 0
         # a block's launches end with its scatter; what precedes block 0 or follows the last block is dense
         geo = dict(geos[min(blk, len(blocks) - 1)], L=lens[i // per_step][min(blk, len(blocks) - 1)])
         bound, amount, *rest = algorithmic_work(name, tag, esz, geo)
-        sym = kernel_symbol(name, tag, dt)
         st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0, "bytes": 0.0})
         st["launches"] += 1
         st["seconds"] += sec
@@ -418,6 +359,8 @@ def run_isolated_gemm(args, torch):
                          "GB/s": round(byts / sec / 1e9, 1), "frac_mfma": round(fl / sec / 1e12 / 2500.0, 4)}
         total_flops += fl
         total_s += sec
+    from vtpack_amd import _lib
+    last_name = _lib.last_kernel()
     ach = total_flops / total_s / 1e12
     return {"metric": "TFLOP/s isolated packed-M GEMM bf16 K=384 @1 MI355X", "value": round(ach, 1),
             "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -427,9 +370,7 @@ def run_isolated_gemm(args, torch):
                        "packed_rows": L},
             "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": 2500.0, "unit": "TFLOP/s",
                          "frac": round(ach / 2500.0, 4),
-                         "kernel": "linear_ws8_kernel<0, true, false, false, false>" if L >= 2048
-                         else "linear_dma_kernel<unsigned short, ...>",
-                         "traffic": None},
+                         "kernel": last_name, "traffic": None},
             "per_n": per_n}
 
 

@@ -46,6 +46,9 @@ extern "C" {
 
 int vtdge_version(void);
 const char *vtdge_last_error(void);
+/* The demangled name of the kernel that the calling thread's latest launch was (the last one, for an entry point
+ * that launches several), as a profiler lists it; "" before the first launch.  For measurement tools. */
+const char *vtdge_last_kernel(void);
 
 /* Router: region mean of the spatial tokens, Linear(C -> S), argmax.
  * Replaces DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75).

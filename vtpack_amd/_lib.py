@@ -52,7 +52,7 @@ SIGNATURES = {
     "vtdge_sparse_attention": [_p, _l, _l, _p, _p, _l, _l, _l, _p, _p, _l, _l, _i, _i, _i, _i, _i, _f, _i, _p],
     "vtdge_batched_sparse_gemm": [_p, _p, _p, _p, _p, _i, _i, _l, _i, _l, _i, _i, _i, _l, _l, _l, _i, _p],
 }
-EXPORTS = ["vtdge_version", "vtdge_last_error"] + list(SIGNATURES)
+EXPORTS = ["vtdge_version", "vtdge_last_error", "vtdge_last_kernel"] + list(SIGNATURES)
 
 _lib = None
 
@@ -86,6 +86,8 @@ def load():
     lib.vtdge_version.argtypes = []
     lib.vtdge_last_error.restype = ctypes.c_char_p
     lib.vtdge_last_error.argtypes = []
+    lib.vtdge_last_kernel.restype = ctypes.c_char_p
+    lib.vtdge_last_kernel.argtypes = []
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _i
@@ -108,6 +110,25 @@ def call(name, *args, tag=None):
     if rc != 0:
         msg = lib.vtdge_last_error().decode("utf-8", "replace")
         raise VtdgeError(f"{name} failed ({rc}): {msg}")
+
+
+def last_kernel():
+    """Name of the kernel the latest libvtdge launch of this thread was, as rocprofv3 lists it (without the
+    namespace and the argument list)."""
+    name = load().vtdge_last_kernel().decode("utf-8", "replace")
+    if name.startswith("void "):
+        name = name[5:]
+    depth, cut = 0, len(name)
+    for i, ch in enumerate(name):            # the argument list opens at the first '(' outside the template brackets
+        if ch == "<":
+            depth += 1
+        elif ch == ">":
+            depth -= 1
+        elif ch == "(" and depth == 0:
+            cut = i
+            break
+    name = name[:cut]
+    return name[len("vtdge::"):] if name.startswith("vtdge::") else name
 
 
 def dtype_code(t):

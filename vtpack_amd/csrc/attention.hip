@@ -235,6 +235,7 @@ static int launch_attention(const void *q, int64_t q_rs, int64_t q_hs, const voi
     auto kern = sparse_attention_kernel<T, D>;
     VT_RESERVE_LDS(kern, lds, "sparse_attention");
     dim3 grid((unsigned)((int64_t)B * qchunks), (unsigned)h), block(256);
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<grid, block, lds, st>>>((const T *)q, q_rs, q_hs, (const T *)k, (const T *)v, kv_bs, kv_ts, kv_hs, offsets,
                                    (T *)out, o_rs, o_hs, n, qchunks, scale);
     return check_launch("sparse_attention");

@@ -625,6 +625,7 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
     case NB: {                                                                                                     \
         auto kern_p = sparse_attention_bf16_d64_pipelined_kernel<NB>;                                              \
         VT_RESERVE_LDS(kern_p, 160 * 1024, "sparse_attention");                                                    \
+        note_kernel(reinterpret_cast<const void *>(kern_p)),                                                        \
         kern_p<<<grid_p, block_p, lds_p, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v, \
                                                kv_bs, kv_ts, kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, scale,  \
                                                items, h);                                                          \
@@ -649,6 +650,7 @@ int launch_attention_bf16_d64(const void *q, int64_t q_rs, int64_t q_hs, const v
     VT_RESERVE_LDS(kern, lds, "sparse_attention");
     const int items = B * h;
     dim3 grid((unsigned)(ceil_div(items, 8) * 8 * qchunks)), block(AQ * 2);
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<grid, block, lds, st>>>((const bf16_t *)q, q_rs, q_hs, (const bf16_t *)k, (const bf16_t *)v, kv_bs, kv_ts,
                                    kv_hs, offsets, (bf16_t *)out, o_rs, o_hs, n, qchunks, scale, items, h);
     return check_launch("sparse_attention");

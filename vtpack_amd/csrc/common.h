@@ -14,6 +14,7 @@ namespace vtdge {
 // ---------------------------------------------------------------- errors
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+void note_kernel(const void *host_function);      // called just before every launch (see vtdge_last_kernel)
 int compute_units();      // of the current device (256 on an MI355X)
 
 #define VT_REQUIRE(cond, code, ...)  \

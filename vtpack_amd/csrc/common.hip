@@ -1,5 +1,7 @@
 // Error plumbing shared by every entry point of libvtdge.
 #include "common.h"
+#include <cxxabi.h>
+#include <stdlib.h>
 
 namespace vtdge {
 
@@ -11,6 +13,27 @@ void set_error(const char *fmt, ...)
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+// The kernel of the latest launch made from this thread, for tools that want to tell a caller's entry points from
+// the kernels a profiler lists (vtdge_last_kernel).  Only the pointer is kept at launch time; the name is looked up
+// and demangled when somebody asks.
+static thread_local const void *last_kernel_fn = nullptr;
+static thread_local char last_kernel_name[512];
+
+void note_kernel(const void *host_function) { last_kernel_fn = host_function; }
+
+extern "C" const char *vtdge_last_kernel(void)
+{
+    last_kernel_name[0] = 0;
+    if (last_kernel_fn == nullptr) return last_kernel_name;
+    const char *mangled = hipKernelNameRefByPtr(last_kernel_fn, nullptr);
+    if (mangled == nullptr) return last_kernel_name;
+    int status = 1;
+    char *plain = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
+    snprintf(last_kernel_name, sizeof(last_kernel_name), "%s", status == 0 && plain ? plain : mangled);
+    free(plain);
+    return last_kernel_name;
 }
 
 int check_launch(const char *what)

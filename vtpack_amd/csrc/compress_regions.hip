@@ -274,6 +274,7 @@ extern "C" int vtdge_compress_regions(const void *x, const int64_t *indices, con
     dim3 grid((unsigned)ceil_div(regions, 4)), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, RECF)                                                                                         \
+    note_kernel(reinterpret_cast<const void *>(compress_regions_kernel<T, RECF>)),                                 \
     compress_regions_kernel<T, RECF><<<grid, block, 0, st>>>((const T *)x, indices, splits, counts, (T *)comp,     \
                                                              (u32x4 *)records, patches, capacity_rows, offsets,    \
                                                              lengths, region_rows, B, H, W, C, extra, S, records_eps)

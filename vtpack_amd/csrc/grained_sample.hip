@@ -1266,6 +1266,7 @@ extern "C" int vtdge_router(const void *x, const void *weight, const void *bias,
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, RS, GS)                                                                                     \
+    note_kernel(reinterpret_cast<const void *>(router_kernel<T, RS, GS>)),                                        \
     router_kernel<T, RS, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)gate, \
                                                      indices, B, H, W, C, extra, R, S)
 #define VT_REGION(T, GS) \
@@ -1303,6 +1304,7 @@ extern "C" int vtdge_router_layernorm(const void *x, const void *weight, const v
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, RS, GS)                                                                                  \
+    note_kernel(reinterpret_cast<const void *>(router_kernel<T, RS, GS, true>)),                              \
     router_kernel<T, RS, GS, true><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias,  \
                                                            (T *)gate, indices, B, H, W, C, extra, R, S,       \
                                                            (const T *)ln_weight, (const T *)ln_bias, ln_eps,  \
@@ -1333,21 +1335,26 @@ extern "C" int vtdge_index_to_patch(const int64_t *indices, const int64_t *split
     hipStream_t st = (hipStream_t)stream;
     if (patches != nullptr && (int64_t)B * Hr * Wr <= 16384) {
         // small batches: one launch, every sample's workgroup sums the counts before it on its own
+        note_kernel(reinterpret_cast<const void *>(patch_write_kernel<true>));
         patch_write_kernel<true><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
                                                     capacity_rows, 0);
         return check_launch("index_to_patch");
     }
     if (patches != nullptr && B <= 4096) {
         // a wave per sample counts, then every sample's workgroup sums the lengths before it (a few KB)
+        note_kernel(reinterpret_cast<const void *>(patch_count_kernel));
         patch_count_kernel<<<(B + 3) / 4, 256, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, lengths);
         if (int rc = check_launch("index_to_patch(count)")) return rc;
+        note_kernel(reinterpret_cast<const void *>(patch_write_kernel<false>));
         patch_write_kernel<false><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
                                                      capacity_rows, 1);
         return check_launch("index_to_patch(write)");
     }
+    note_kernel(reinterpret_cast<const void *>(patch_count_scan_kernel));
     patch_count_scan_kernel<<<1, 1024, 0, st>>>(indices, splits, B, Hr * Wr, S, extra, offsets, lengths);
     if (int rc = check_launch("index_to_patch(count+scan)")) return rc;
     if (patches != nullptr) {
+        note_kernel(reinterpret_cast<const void *>(patch_write_kernel<false>));
         patch_write_kernel<false><<<B, 256, 0, st>>>(indices, splits, offsets, lengths, Hr, Wr, S, R, extra, patches,
                                                      capacity_rows, 0);
         return check_launch("index_to_patch(write)");
@@ -1371,6 +1378,7 @@ extern "C" int vtdge_index_to_patch_dense(const int64_t *splits_host, int B, int
         per += sp.ps[s] * sp.ps[s] * Hr * Wr;
     }
     const int64_t total = (int64_t)B * per;
+    note_kernel(reinterpret_cast<const void *>(patch_dense_kernel));
     patch_dense_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(sp, B, Hr, Wr, R, extra,
                                                                                         per, patches);
     return check_launch("index_to_patch_dense");
@@ -1395,6 +1403,7 @@ extern "C" int vtdge_compress(const void *x, const int64_t *patches, const int64
     dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, LNF, GS, NIT)                                                                                  \
+    note_kernel(reinterpret_cast<const void *>(compress_kernel<T, LNF, GS, NIT>)),                                  \
     compress_kernel<T, LNF, GS, NIT><<<grid, block, 0, st>>>((const T *)x, patches, rows_dev, rows, (T *)out,       \
                                                              (T *)ln_out, (const T *)ln_weight, (const T *)ln_bias, \
                                                              ln_eps, N, C, W, extra)
@@ -1428,6 +1437,7 @@ extern "C" int vtdge_decompress(const void *in, const void *sub, const int64_t *
     dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, SUBF, ADDF, GS)                                                                              \
+    note_kernel(reinterpret_cast<const void *>(decompress_kernel<T, SUBF, ADDF, GS>)),                             \
     decompress_kernel<T, SUBF, ADDF, GS><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev, \
                                                                  rows, (const T *)ref, (T *)out, N, C, W, extra)
 #define VT_DISPATCH(T, GS)                                       \
@@ -1469,6 +1479,7 @@ extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const
     dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK * (WAVE / gs))), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define VT_LAUNCH(T, SUBF, GS)                                                                                      \
+    note_kernel(reinterpret_cast<const void *>(decompress_ln_kernel<T, SUBF, GS>)),                                 \
     decompress_ln_kernel<T, SUBF, GS><<<grid, block, 0, st>>>((const T *)in, (const T *)sub, patches, rows_dev,     \
                                                               rows, (const T *)ref, (T *)out, (T *)ln_out,          \
                                                               (const T *)ln_weight, (const T *)ln_bias, ln_eps, N,  \
@@ -1517,6 +1528,7 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
                    "decompress_router: statistics records are written for bf16 rows of 264 to 512 channels (C=%d)", C);
         VT_REQUIRE(aligned16(out_records), VTDGE_ERR_ARG, "decompress_router: records must be 16-byte aligned");
 #define VT_STAT(SUBF)                                                                                                \
+    note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<bf16_t, WAVE, SUBF, true>)),                  \
     decompress_route_kernel<bf16_t, WAVE, SUBF, true><<<grid, block, 0, st>>>(                                       \
         (const bf16_t *)in, (const bf16_t *)sub, cur_indices, splits, offsets, (const bf16_t *)ref, (bf16_t *)out,   \
         (const bf16_t *)next_weight, (const bf16_t *)next_bias, (bf16_t *)next_gate, next_indices, B, H, W, C, extra, \
@@ -1526,6 +1538,7 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
         return check_launch("decompress_router");
     }
 #define VT_LAUNCH2(T, GS, SUBF)                                                                                    \
+    note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<T, GS, SUBF>)),                             \
     decompress_route_kernel<T, GS, SUBF><<<grid, block, 0, st>>>(                                                  \
         (const T *)in, (const T *)sub, cur_indices, splits, offsets, (const T *)ref, (T *)out,                     \
         (const T *)next_weight, (const T *)next_bias, (T *)next_gate, next_indices, B, H, W, C, extra, S, S2,      \
@@ -1560,6 +1573,7 @@ extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *w
                "router_stats: operands must be 16-byte aligned");
     const int64_t regions = (int64_t)B * (H / R) * (W / R);
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
+    note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<bf16_t, WAVE, false, true, false>));
     decompress_route_kernel<bf16_t, WAVE, false, true, false><<<grid, block, 0, (hipStream_t)stream>>>(
         (const bf16_t *)front_rows, nullptr, nullptr, splits, nullptr, (const bf16_t *)x, (bf16_t *)x,
         (const bf16_t *)weight, (const bf16_t *)bias, (bf16_t *)gate, indices, B, H, W, C, extra, S, S,
@@ -1584,6 +1598,7 @@ extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bi
     hipStream_t st = (hipStream_t)stream;
     const int nit = (int)ceil_div(C / vec, WAVE);
 #define VT_LAUNCH(T, NIT, GS)                                                                                        \
+    note_kernel(reinterpret_cast<const void *>(layernorm_kernel<T, NIT, GS>)),                                       \
     layernorm_kernel<T, NIT, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
                                                          rows_dev, rows, C, eps)
 #define VT_GROUP(T)                                                                                       \
@@ -1612,6 +1627,7 @@ extern "C" int vtdge_layernorm_stats(const void *x, void *records, const int64_t
     hipStream_t st = (hipStream_t)stream;
     const int nit = (int)ceil_div(C / 8, WAVE);
 #define VT_LAUNCH(NIT, GS) \
+    note_kernel(reinterpret_cast<const void *>(layernorm_stats_kernel<NIT, GS>)), \
     layernorm_stats_kernel<NIT, GS><<<grid, block, 0, st>>>((const bf16_t *)x, (u32x4 *)records, rows_dev, rows, C, eps)
     if (gs == 64) { if (nit == 1) VT_LAUNCH(1, 64); else if (nit == 2) VT_LAUNCH(2, 64); else VT_LAUNCH(3, 64); }
     else if (gs == 32) VT_LAUNCH(1, 32); else if (gs == 16) VT_LAUNCH(1, 16); else VT_LAUNCH(1, 8);

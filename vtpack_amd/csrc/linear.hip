@@ -158,6 +158,7 @@ static int launch_linear(const void *A, int64_t lda, const void *W, const void *
     do {                                                                                                        \
         auto kern = linear_kernel<T, ACT, HB, HR>;                                                              \
         VT_RESERVE_LDS(kern, lds, "linear");                                                                    \
+        note_kernel(reinterpret_cast<const void *>(kern)),                                                      \
         kern<<<grid, block, lds, st>>>((const T *)A, lda, (const T *)W, (const T *)bias, (const T *)res, ldr,   \
                                        (T *)out, ldo, rows_dev, rows, N, K);                                    \
     } while (0)
@@ -283,6 +284,7 @@ extern "C" int vtdge_linear_prepack(const void *W, int N, int K, int dtype, void
     VT_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)packed & 15) == 0, VTDGE_ERR_ARG,
                "linear_prepack: W and packed must be 16-byte aligned");
     const int64_t units = (int64_t)N * K / 8;
+    note_kernel(reinterpret_cast<const void *>(linear_prepack_kernel));
     linear_prepack_kernel<<<(unsigned)ceil_div(units, 256), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t *)W, (u32x4 *)packed, N, K, layout);
     return check_launch("linear_prepack");
@@ -324,6 +326,7 @@ extern "C" int vtdge_layernorm_fold(const void *W, const void *bias, const void 
     VT_REQUIRE(N > 0 && K > 0, VTDGE_ERR_ARG, "layernorm_fold: bad sizes N=%d K=%d", N, K);
     VT_REQUIRE(dtype == VTDGE_BF16, VTDGE_ERR_UNSUPPORTED, "layernorm_fold: built for bf16 weights only");
     VT_REQUIRE(((uintptr_t)col_records & 15) == 0, VTDGE_ERR_ARG, "layernorm_fold: records must be 16-byte aligned");
+    note_kernel(reinterpret_cast<const void *>(layernorm_fold_kernel));
     layernorm_fold_kernel<<<(unsigned)ceil_div(N, 4), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)ln_weight, (const bf16_t *)ln_bias, (bf16_t *)W_folded,
         (u32x4 *)col_records, N, K);

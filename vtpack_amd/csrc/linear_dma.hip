@@ -357,6 +357,7 @@ static int go(const LinArgs &a, const PatchGeom &pg = PatchGeom{0, 0, 0, 0, 0, 0
     int64_t wgs_per_xcd = 32 * WGS_PER_CU;
     if (wgs_per_xcd > tiles_per_xcd) wgs_per_xcd = tiles_per_xcd;
     dim3 grid((unsigned)(wgs_per_xcd * 8)), block(NW * 64);
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<grid, block, lds, a.st>>>((const T *)a.A, a.lda, (const T *)a.W, (const T *)a.bias, (const T *)a.res,
                                      a.ldr, (T *)a.out, a.ldo, a.rows_dev, a.rows, a.N, a.K, pg);
     return check_launch("linear");

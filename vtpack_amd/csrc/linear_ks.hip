@@ -376,6 +376,7 @@ static int go_ks(const void *A, int64_t lda, const void *W, const void *Wp, cons
     const int64_t tiles_m = ceil_div(rows, 16);
     if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
     dim3 grid((unsigned)(P * groups)), block(256);
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
                                    ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp);
     return check_launch("linear");

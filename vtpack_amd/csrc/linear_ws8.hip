@@ -529,6 +529,7 @@ static int go_ws8(const void *A, int64_t lda, const void *W, const void *Wp, con
     const int64_t tiles_m = ceil_div(rows, 32);
     if (P > tiles_m) P = (int)((tiles_m + 7) & ~7);
     dim3 grid((unsigned)(P * groups)), block(512);
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<grid, block, lds, st>>>((const bf16_t *)A, lda, (const bf16_t *)W, (const bf16_t *)bias, (const bf16_t *)res,
                                    ldr, (bf16_t *)out, ldo, rows_dev, rows, groups, P, (const u32x4 *)Wp,
                                    (const u32x4 *)lnrec, (const u32x4 *)lnw, (u32x4 *)stat_out, stat_eps);
@@ -587,6 +588,7 @@ int launch_linear_ws8_ln_pair(const void *A0, int64_t lda0, const void *lnrec0, 
     // one workgroup per CU in units of 8 (one per XCD); at least one unit per column group of either problem
     int units = compute_units() / 8;
     if (units < a.groups + b.groups) units = a.groups + b.groups;
+    note_kernel(reinterpret_cast<const void *>(kern));
     kern<<<dim3((unsigned)(units * 8)), dim3(512), lds, st>>>(a, b);
     return check_launch("linear");
 }

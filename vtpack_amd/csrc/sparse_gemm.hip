@@ -150,10 +150,12 @@ extern "C" int vtdge_batched_sparse_gemm(const void *a, const void *b, const int
     const bool vec_a = (ka * esz) % 16 == 0 && ((uintptr_t)a & 15) == 0;
     const bool vec_b = (kb * esz) % 16 == 0 && ((uintptr_t)b & 15) == 0;
     if (dtype == VTDGE_F32)
+        note_kernel(reinterpret_cast<const void *>(sparse_gemm_kernel<float>)),
         sparse_gemm_kernel<float><<<grid, block, 0, st>>>((const float *)a, (const float *)b, a_offsets, b_offsets,
                                                           (float *)out, h, La, ka, Lb, kb, trans_a, trans_b, out_rows,
                                                           out_cols, (int)tiles_m, (int)tiles_n, vec_a, vec_b);
     else
+        note_kernel(reinterpret_cast<const void *>(sparse_gemm_kernel<bf16_t>)),
         sparse_gemm_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t *)a, (const bf16_t *)b, a_offsets,
                                                            b_offsets, (bf16_t *)out, h, La, ka, Lb, kb, trans_a,
                                                            trans_b, out_rows, out_cols, (int)tiles_m, (int)tiles_n, vec_a, vec_b);
