@@ -254,6 +254,24 @@ def test_deit_small_bf16_model_on_the_weight_stationary_kernels(dev):
     assert_close(got.float(), want, torch.bfloat16, "DeiT-S+DGE bf16 logits, batch 8")
 
 
+@pytest.mark.parametrize("factory,heads", [("deit_dge_s124_base_patch16_256", 12), ("deit_dge_s124_tiny_patch16_256", 3)])
+def test_deit_other_widths_bf16_model(dev, factory, heads):
+    """The other widths the reference ships (DeiT-Base: 768 channels, 12 heads; DeiT-Ti: 192 channels, 3 heads;
+    vtpack/models/dge/deit_dge.py:302-329) in bf16: the streaming Linear and the row-wise sampling kernels instead of
+    the weight-stationary ones, same bar as DeiT-S."""
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model(factory, dev, torch.bfloat16, seed=6)
+    img = synthetic_images(2, 256, seed=8, dtype=torch.bfloat16)
+    with torch.no_grad():
+        got = m(img.to(dev))
+    want, traces = forced_reference(m, img.float(), heads, 12)
+    for blk, tr in zip(m.blocks, traces):
+        assert torch.equal(blk.dge.states["patches"].cpu(), tr["patches"])
+        assert torch.equal(blk.dge.states["batches"], tr["lengths"])
+    _assert_bf16_gates_differ_only_at_near_ties(m, traces, 0.95)
+    assert_close(got.float(), want, torch.bfloat16, f"{factory} bf16 logits")
+
+
 def test_high_res_geometry(dev):
     """Config 5 geometry (512 px: 1024 tokens + cls, 64 regions, KV length 1025) on a 2-layer fp32 model."""
     from vtpack_amd.models.dge.deit_dge import VisionTransformer

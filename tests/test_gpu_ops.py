@@ -411,6 +411,34 @@ def test_linear_weight_stationary(dev, M, N, epi):
     assert float((err / want.abs().clamp_min(4)).max()) <= 2 ** -7, f"weight-stationary linear {epi} (relative)"
 
 
+@pytest.mark.parametrize("N", [384, 1152, 1536])
+def test_linear_on_skewed_segments(dev, N):
+    """The isolated grouped GEMM of the benchmark (bf16, K = 384, 256 samples whose query counts follow a seeded
+    skewed gate mix with a heavy tail, clipped to [16, 256]; A ~ N(0, 1), W ~ N(0, 0.02)): the packed rows of all
+    segments against one shared weight, checked against fp64 on every row, with the live row count on the device."""
+    from vtpack_amd import ops
+    r = np.random.RandomState(0)
+    p_fine = np.clip(r.beta(0.6, 2.0, size=256), 0, 1)
+    lengths = np.clip(np.array([1 + int(r.choice([16, 4, 1], size=16, p=[pf, (1 - pf) * 0.4, (1 - pf) * 0.6]).sum())
+                                for pf in p_fine]), 16, 256)
+    L, K = int(lengths.sum()), 384
+    assert L == 21911                                    # the benchmark's segments
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn((L, K), generator=g).bfloat16().to(dev)
+    w = (torch.randn((N, K), generator=g) * 0.02).bfloat16().to(dev)
+    bias = (torch.randn(N, generator=g) * 0.02).bfloat16().to(dev)
+    cap = torch.zeros((L + 4096, K), dtype=torch.bfloat16, device=dev)
+    cap[:L] = a
+    out = ops.linear(cap, w, bias, rows_dev=torch.tensor([L], dtype=torch.int64, device=dev))
+    want = a.double() @ w.double().T + bias.double()
+    assert abs_err(out[:L], want) <= BF16_ABS
+    # segment boundaries mean nothing to a Linear with shared weights: any one segment alone gives the same rows
+    off = np.concatenate([[0], np.cumsum(lengths)])
+    big = int(lengths.argmax())
+    alone = ops.linear(a[off[big]:off[big + 1]].contiguous(), w, bias)
+    assert abs_err(alone, want[off[big]:off[big + 1]]) <= BF16_ABS
+
+
 def test_linear_weight_stationary_device_rows(dev):
     from vtpack_amd import ops
     M, N, K, live = 6000, 768, 384, 4999
