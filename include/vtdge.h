@@ -194,6 +194,12 @@ int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t 
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */
 int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out, const int64_t *rows_dev,
                     int64_t rows, int C, float eps, int dtype, void *stream);
+/* The same for input rows that lie in groups: row r is x + (r / x_group_rows) * x_group_stride + (r % x_group_rows) * C
+ * (elements); out [rows, C] is dense.  The final norm of a model only on the rows the classifier reads - the class
+ * (and distillation) tokens, the first rows of every sample (vtpack/models/dge/deit_dge.py:283-285 with :288-299) -
+ * without a gathered copy of them: x_group_rows = extra, x_group_stride = N * C. */
+int vtdge_layernorm_rows(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight, const void *bias,
+                         void *out, int64_t rows, int C, float eps, int dtype, void *stream);
 
 /* Packed-M Linear: out[m, n] = act(sum_k A[m,k] * W[n,k] + bias[n]) + residual[m,n].
  * The M dimension is the packed query set of all samples (weights are shared),

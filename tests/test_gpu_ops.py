@@ -346,6 +346,18 @@ def test_layernorm(dev, dtype, rows, C):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,N,C,count", [(256, 257, 384, 1), (5, 66, 192, 2), (3, 17, 768, 17), (9, 10, 64, 3)])
+def test_layernorm_of_the_front_rows(dev, dtype, B, N, C, count):
+    """The final norm on the class-token rows only, read in place: the same bits as LayerNorm of a copy of the slice."""
+    from vtpack_amd import ops
+    x = _t(randn(131, B, N, C) * 1.5 + 0.3, dev, dtype)
+    w, b = _t(randn(132, C) * 0.2 + 1, dev, dtype), _t(randn(133, C) * 0.1, dev, dtype)
+    got = ops.layernorm_front_rows(x, count, w, b, 1e-6)
+    assert got.shape == (B, count, C)
+    assert torch.equal(got, ops.layernorm(x[:, :count, :].contiguous(), w, b, 1e-6))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 192, 192), (904, 576, 192), (257, 384, 384), (1000, 1536, 384),
                                      (300, 384, 1536), (129, 1000, 192), (64, 72, 40)])
 @pytest.mark.parametrize("epi", ["plain", "bias", "bias_gelu", "bias_res"])

@@ -1109,7 +1109,7 @@ template <typename T, int NIT, int GS>   // NIT = 16-byte vectors per lane = cei
 __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                          const T *__restrict__ bsrc, T *__restrict__ out,
                                                          const int64_t *__restrict__ rows_dev, int64_t rows, int C,
-                                                         float eps)
+                                                         float eps, int64_t x_group_stride, int x_group_rows)
 {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & (GS - 1);
@@ -1124,8 +1124,10 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
             const int v = it * WAVE + lane;
-            if (v < nvec && row0 + r < live)
-                raw[r][it] = *reinterpret_cast<const u32x4 *>(x + (row0 + r) * (int64_t)C + v * VEC);
+            // input rows come in groups of x_group_rows dense rows, the groups x_group_stride elements apart
+            const int64_t rr = row0 + r;
+            const int64_t src = x_group_rows > 0 ? (rr / x_group_rows) * x_group_stride + (rr % x_group_rows) * C : rr * C;
+            if (v < nvec && rr < live) raw[r][it] = *reinterpret_cast<const u32x4 *>(x + src + v * VEC);
         }
     float ww[NIT][VEC], bb[NIT][VEC];
 #pragma unroll
@@ -1581,8 +1583,30 @@ extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *w
     return check_launch("router_stats");
 }
 
+static int layernorm_launch(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight,
+                            const void *bias, void *out, const int64_t *rows_dev, int64_t rows, int C, float eps,
+                            int dtype, void *stream);
+
 extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,
                                const int64_t *rows_dev, int64_t rows, int C, float eps, int dtype, void *stream)
+{
+    return layernorm_launch(x, 0, 0, weight, bias, out, rows_dev, rows, C, eps, dtype, stream);
+}
+
+extern "C" int vtdge_layernorm_rows(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight,
+                                    const void *bias, void *out, int64_t rows, int C, float eps, int dtype,
+                                    void *stream)
+{
+    VT_REQUIRE(x_group_rows > 0 && x_group_stride >= (int64_t)x_group_rows * C, VTDGE_ERR_ARG,
+               "layernorm_rows: groups of %d rows %lld elements apart overlap", x_group_rows, (long long)x_group_stride);
+    const int vec = dtype == VTDGE_BF16 ? 8 : 4;
+    VT_REQUIRE(x_group_stride % vec == 0, VTDGE_ERR_ARG, "layernorm_rows: the group stride must keep rows 16-byte aligned");
+    return layernorm_launch(x, x_group_stride, x_group_rows, weight, bias, out, nullptr, rows, C, eps, dtype, stream);
+}
+
+static int layernorm_launch(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight,
+                            const void *bias, void *out, const int64_t *rows_dev, int64_t rows, int C, float eps,
+                            int dtype, void *stream)
 {
     VT_REQUIRE(x && weight && bias && out, VTDGE_ERR_ARG, "layernorm: NULL operand");
     VT_REQUIRE(rows >= 0, VTDGE_ERR_ARG, "layernorm: negative rows");
@@ -1600,7 +1624,7 @@ extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bi
 #define VT_LAUNCH(T, NIT, GS)                                                                                        \
     note_kernel(reinterpret_cast<const void *>(layernorm_kernel<T, NIT, GS>)),                                       \
     layernorm_kernel<T, NIT, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
-                                                         rows_dev, rows, C, eps)
+                                                         rows_dev, rows, C, eps, x_group_stride, x_group_rows)
 #define VT_GROUP(T)                                                                                       \
     do {                                                                                                  \
         if (gs == 64) { if (nit == 1) VT_LAUNCH(T, 1, 64); else if (nit == 2) VT_LAUNCH(T, 2, 64); else VT_LAUNCH(T, 3, 64); } \

@@ -410,7 +410,7 @@ def model_forward(model, images):
     if extra == 0:      # no class token: the classifier sees the mean over all normalised tokens
         return head(model.head, ops.layernorm(x, nrm.weight, nrm.bias, nrm.eps).mean(dim=1))
     # only the rows of the extra tokens are needed after the last block
-    feats = ops.layernorm(x[:, :extra, :], nrm.weight, nrm.bias, nrm.eps)
+    feats = ops.layernorm_front_rows(x, extra, nrm.weight, nrm.bias, nrm.eps)
     if extra == 2:      # class + distillation token: the mean of the two classifiers (deit_dge.py:288-294)
         return (head(model.head, feats[:, 0]) + head(model.head_dist, feats[:, 1])) / 2
     cls = feats[:, 0]

@@ -362,6 +362,22 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
     return out
 
 
+def layernorm_front_rows(x, count, weight, bias, eps=1e-6):
+    """LayerNorm of the first `count` rows of every sample of x [B, N, C] -> [B, count, C], read in place (no copy of
+    the slice): the model's final norm on the class-token rows only."""
+    _need_gpu(x, weight, bias)
+    if x.dim() != 3 or not x.is_contiguous() or not 0 < count <= x.shape[1]:
+        raise ValueError("layernorm_front_rows takes contiguous [B, N, C] tokens and 0 < count <= N")
+    B, N, C = x.shape
+    _check_like(x, weight=weight, bias=bias)
+    _check_vector("weight", weight, C)
+    _check_vector("bias", bias, C)
+    out = torch.empty((B, count, C), dtype=x.dtype, device=x.device)
+    call("vtdge_layernorm_rows", ptr(x), N * C, count, ptr(_contig(weight)), ptr(_contig(bias)), ptr(out), B * count, C,
+         float(eps), dtype_code(x), stream_ptr(), tag=("layernorm", False, B * count, C))
+    return out
+
+
 PACK_WEIGHTS = True     # module switch (tests compare the two paths)
 _pack_epoch = 0         # bumped by invalidate_packed(): every packed copy made before is stale
 
