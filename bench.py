@@ -133,6 +133,12 @@ def algorithmic_work(name, tag, esz, geo):
         # the scatter-back's bytes: routing the next block reads nothing more (gate indices in, logits out: KBs)
         return "hbm", ((2 if tag[1] else 1) * L * C * esz + 2 * B * N * C * esz + 16 * B * geo["regions"]
                        + (32 * B * N if tag[4] else 0))
+    if name == "vtdge_decompress_router_compress":
+        # the scatter-back's bytes plus the next block's queries with their records and descriptors (the tokens the
+        # kernel reads back are the ones it has just written)
+        Ln = geo["L_next"]
+        return "hbm", ((2 if tag[1] else 1) * L * C * esz + 2 * B * N * C * esz + 16 * B * geo["regions"]
+                       + 32 * B * N + Ln * C * esz + (32 * Ln if tag[3] else 0) + 32 * Ln)
     if name == "vtdge_decompress_layernorm":
         # the scatter-back plus one more write of every token (the next block's first LayerNorm)
         return "hbm", (2 if tag[1] else 1) * L * C * esz + 32 * L + 3 * B * N * C * esz
@@ -250,14 +256,16 @@ def run_model_workload(args, torch):
         if i % per_step == 0:
             blk = 0
         # a block's launches end with its scatter; what precedes block 0 or follows the last block is dense
-        geo = dict(geos[min(blk, len(blocks) - 1)], L=lens[i // per_step][min(blk, len(blocks) - 1)])
+        at = min(blk, len(blocks) - 1)
+        geo = dict(geos[at], L=lens[i // per_step][at], L_next=lens[i // per_step][min(at + 1, len(blocks) - 1)])
         bound, amount, *rest = algorithmic_work(name, tag, esz, geo)
         st = stats.setdefault(sym, {"bound": bound, "launches": 0, "seconds": 0.0, "work": 0.0, "bytes": 0.0})
         st["launches"] += 1
         st["seconds"] += sec
         st["work"] += amount
         st["bytes"] += rest[0] if rest else 0.0
-        if name in ("vtdge_decompress", "vtdge_decompress_router", "vtdge_decompress_layernorm"):
+        if name in ("vtdge_decompress", "vtdge_decompress_router", "vtdge_decompress_router_compress",
+                    "vtdge_decompress_layernorm"):
             blk += 1
     kernels = {}
     for sym, st in stats.items():

@@ -153,6 +153,33 @@ int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_
                             const int32_t *region_rows, const uint8_t *cur_counts, int B, int H, int W, int C,
                             int extra, int R, int S, int S2, int dtype, void *stream);
 
+/* vtdge_decompress_router that goes on to pack the NEXT block's queries from the tokens it has just written: the
+ * scatter-back of one block (vtpack/layers/dge.py:87-112), the next block's router (:145-150, :75) and the next
+ * block's index->patch + compress (:76-79) in one launch, i.e. vtdge_decompress_router followed by
+ * vtdge_compress_regions without a second pass over the tokens.  All outputs are bit-identical to those two calls.
+ *   next_comp [capacity_rows, C], next_comp_records [capacity_rows, 16] bf16 with next_records_eps,
+ *   next_patches (nullable) [capacity_rows, 4], next_offsets [B+1], next_region_rows (nullable) int32 [regions]:
+ *   as vtdge_compress_regions writes comp, records, patches, offsets and region_rows (lengths are the differences
+ *   of the offsets and are not written)
+ *   workspace: vtdge_decompress_router_compress_workspace(B, H, W, R) bytes of device memory, 8-byte aligned, all
+ *   zero when the kernel starts (clear_workspace != 0: the call clears it first with a small fill kernel; a caller
+ *   that keeps one slice per block can clear them all at once instead).  The workgroups hand the running number of
+ *   queries along through it (one 64-bit word each); word 0 is raised to 1 if a workgroup gave up waiting for the
+ *   ones before it, in which case rows are missing from next_comp and next_offsets[B] exceeds capacity_rows.
+ * bf16 rows of 264 to 512 channels, R = 4, splits out of {1, 2, 4}, the regions a multiple of 4 up to 65536, the
+ * next router with its splits and count bytes, out_records present; VTDGE_ERR_UNSUPPORTED otherwise. */
+int64_t vtdge_decompress_router_compress_workspace(int B, int H, int W, int R);
+int vtdge_decompress_router_compress(const void *in, const void *sub, const int64_t *cur_indices,
+                                     const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
+                                     const void *next_weight, const void *next_bias, void *next_gate,
+                                     int64_t *next_indices, void *out_records, float records_eps,
+                                     const int64_t *next_splits, uint8_t *next_counts, const int32_t *region_rows,
+                                     const uint8_t *cur_counts, void *next_comp, void *next_comp_records,
+                                     float next_records_eps, int64_t *next_patches, int64_t capacity_rows,
+                                     int64_t *next_offsets, int32_t *next_region_rows, void *workspace,
+                                     int64_t workspace_bytes, int clear_workspace, int B, int H, int W, int C,
+                                     int extra, int R, int S, int S2, int dtype, void *stream);
+
 /* The router of a model's FIRST block together with the statistics records of all its tokens (no scatter-back
  * precedes it that could leave them): vtdge_router and vtdge_layernorm_stats in one pass over x, i.e.
  * DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75) and the statistics half of norm1

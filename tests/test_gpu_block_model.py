@@ -244,8 +244,10 @@ def test_deit_small_bf16_model_on_the_weight_stationary_kernels(dev):
         _lib.timer = None
     assert names.names.count("vtdge_linear_layernorm") == 12 and names.names.count("vtdge_linear_layernorm_pair") == 12
     assert names.names.count("vtdge_linear_stats") == 12
-    assert names.names.count("vtdge_decompress_router") == 11 and names.names.count("vtdge_layernorm_rows") == 1
-    assert names.names.count("vtdge_compress_regions") == 12 and names.names.count("vtdge_index_to_patch") == 0
+    # the first block packs its own queries; every scatter-back but the last also packs the next block's
+    assert names.names.count("vtdge_decompress_router_compress") == 11 and names.names.count("vtdge_decompress") == 1
+    assert names.names.count("vtdge_decompress_router") == 0 and names.names.count("vtdge_layernorm_rows") == 1
+    assert names.names.count("vtdge_compress_regions") == 1 and names.names.count("vtdge_index_to_patch") == 0
     want, traces = forced_reference(m, img.float(), 6, 12)
     for blk, tr in zip(m.blocks, traces):
         assert torch.equal(blk.dge.states["patches"].cpu(), tr["patches"])

@@ -357,6 +357,67 @@ def test_scatter_records_refused_for_other_rows(dev):
     assert not ops.fits_scatter_stats(x) and not ops.fits_scatter_stats(x.float())
 
 
+# ----------------------------------------------------------------------------- the scatter-back that packs the
+# next block's queries (vtpack/layers/dge.py:87-112, then :145-150, :75-79 of the next block) against the two kernels
+# it stands for: every output bit for bit
+@pytest.mark.parametrize("B,H,W,Cc,extra,with_sub", [(8, 16, 16, 384, 1, True), (4, 32, 32, 384, 2, True),
+                                                     (4, 8, 8, 512, 0, False), (2, 8, 8, 264, 1, True),
+                                                     (3, 8, 16, 384, 1, True), (256, 16, 16, 384, 1, True),
+                                                     (64, 32, 32, 384, 0, True)])
+def test_scatter_back_packs_the_next_queries(dev, B, H, W, Cc, extra, with_sub):
+    from vtpack_amd import ops
+    N = extra + H * W
+    g = torch.Generator().manual_seed(B + Cc)
+    idx = torch.from_numpy(random_indices(B, B, H // 4, W // 4)).to(dev)
+    splits = torch.tensor(SPLITS, dtype=torch.int64, device=dev)
+    next_splits = torch.tensor(SPLITS[::-1], dtype=torch.int64, device=dev)
+    x = (torch.randn(B, N, Cc, generator=g) * 2 + 3 * torch.randn(B, N, 1, generator=g)).bfloat16().to(dev)
+    assert ops.fits_pack_next(x, H, W, 4, SPLITS)
+    comp, _, patches, offsets, lengths, rrows = ops.compress_regions(x, idx, splits, H, W, 4, want_region_rows=True)
+    q = torch.randn(B * N, Cc, generator=g).bfloat16().to(dev)
+    wgt = (torch.randn(3, Cc, generator=g) * 0.3).bfloat16().to(dev)
+    bias = (torch.randn(3, generator=g) * 0.3).bfloat16().to(dev)
+    sub = comp if with_sub else None
+    want = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt, next_bias=bias,
+                                 stats_eps=EPS, next_splits=next_splits)
+    w_out, w_gate, w_idx, w_rec, w_cnt = want
+    assert len(set(w_idx.reshape(-1).tolist())) >= 2            # a mix of splits
+    w_comp, w_crec, w_pat, w_off, w_len, w_rows = ops.compress_regions(
+        w_out, w_idx, next_splits, H, W, 4, counts=w_cnt, stats_eps=2 * EPS, want_region_rows=True)
+    total = int(w_off[B])
+    words = ops.pack_next_workspace_words(B, H, W, 4)
+    ws = torch.zeros(words + 3, dtype=torch.int64, device=dev)
+    for trial in range(4):
+        kw = dict(workspace=ws) if trial % 2 else {}
+        if trial % 2:
+            ws.zero_()
+        got = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt, next_bias=bias,
+                                    stats_eps=EPS, next_splits=next_splits, pack_next=True, pack_eps=2 * EPS, **kw)
+        out, gate, nidx, rec, cnt, packed = got
+        assert int(packed["workspace"][0]) == 0
+        assert torch.equal(out, w_out) and torch.equal(gate, w_gate) and torch.equal(nidx, w_idx)
+        assert torch.equal(rec, w_rec) and torch.equal(cnt[:nidx.numel()], w_cnt[:nidx.numel()])
+        assert torch.equal(packed["offsets"], w_off)
+        assert torch.equal(packed["region_rows"], w_rows)
+        assert torch.equal(packed["comp"][:total], w_comp[:total])
+        assert torch.equal(packed["records"][:total], w_crec[:total])
+        assert torch.equal(packed["patches"][:total], w_pat[:total])
+    # the regions' first rows of this block handed over as well
+    got = ops.decompress_router(q, idx, splits, offsets, x, H, W, 4, sub=sub, next_weight=wgt, next_bias=bias,
+                                stats_eps=EPS, next_splits=next_splits, pack_next=True, pack_eps=2 * EPS,
+                                region_rows=rrows, cur_counts=(splits[idx.reshape(-1)] ** 2).to(torch.uint8))
+    assert torch.equal(got[0], w_out) and torch.equal(got[5]["records"][:total], w_crec[:total])
+    assert torch.equal(got[5]["comp"][:total], w_comp[:total]) and torch.equal(got[5]["offsets"], w_off)
+
+
+def test_pack_next_refuses_partial_workgroups(dev):
+    from vtpack_amd import ops
+    x = torch.zeros(3, 1 + 8 * 8, 384, dtype=torch.bfloat16, device=dev)     # 3 * 4 regions: fine
+    assert ops.fits_pack_next(x, 8, 8, 4, SPLITS)
+    x = torch.zeros(3, 1 + 12 * 4, 384, dtype=torch.bfloat16, device=dev)    # 3 * 3 regions
+    assert not ops.fits_pack_next(x, 12, 4, 4, SPLITS)
+
+
 # ----------------------------------------------------------------------------- the model with and without
 def test_model_with_and_without_folded_norms(dev):
     """DeiT-S+DGE, bf16, 256 px, batch 16 (enough rows for the weight-stationary kernels): with the folding on the

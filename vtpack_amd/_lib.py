@@ -34,6 +34,9 @@ SIGNATURES = {
     "vtdge_decompress_layernorm": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_decompress_router": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _p, _i, _i, _i, _i,
                                 _i, _i, _i, _i, _i, _p],
+    "vtdge_decompress_router_compress": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _p,
+                                         _p, _p, _f, _p, _l, _p, _p, _p, _l, _i,
+                                         _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_router_stats": [_p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_compress_regions": [_p, _p, _p, _p, _p, _p, _f, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_layernorm": [_p, _p, _p, _p, _p, _l, _i, _f, _i, _p],
@@ -89,6 +92,8 @@ def load():
     lib.vtdge_last_error.argtypes = []
     lib.vtdge_last_kernel.restype = ctypes.c_char_p
     lib.vtdge_last_kernel.argtypes = []
+    lib.vtdge_decompress_router_compress_workspace.restype = _l
+    lib.vtdge_decompress_router_compress_workspace.argtypes = [_i, _i, _i, _i]
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _i

@@ -7,6 +7,7 @@
 // with fully coalesced 16-byte accesses and narrow rows (C = 64, 128: the
 // first PVT stages) still keep every lane of the wavefront busy.
 #include "common.h"
+#include "region_pack.h"
 #include <type_traits>
 
 namespace vtdge {
@@ -939,21 +940,46 @@ __device__ __forceinline__ void region_read(const T *__restrict__ refp, int W, i
     }
 }
 
+// CHAIN = true: the kernel goes on to pack the NEXT block's queries (what vtdge_compress_regions would do in a launch
+// of its own, reading the tokens back): the wave that has just written a region's tokens and chosen its next split has
+// everything for that but the region's first packed row, which is the number of queries of ALL regions before it.
+// The workgroups pass that number along in launch order through one 64-bit status word each (two flag bits + a
+// count): a workgroup publishes the queries of its four regions ("aggregate"), looks back over the words of the
+// workgroups before it - 64 of them per step, one per lane - until it meets one that already knows its total
+// ("prefix"), adds up what lies between and publishes its own prefix.  A workgroup only ever waits for workgroups
+// with smaller numbers, which were dispatched before it and wait for nobody behind them, so the chain always moves;
+// the wait is bounded all the same (a workgroup that gives up raises the error word and places its rows past the
+// capacity, where nothing is written).  The status words must be zero at launch; nothing else of them is kept.
+struct ChainArgs {
+    bf16_t *comp;                 // [capacity, C] the next block's packed queries
+    u32x4 *comp_records;          // [capacity, 2] their statistics records
+    float comp_eps;
+    int64_t *patches;             // [capacity, 4] (nullable)
+    int64_t capacity;
+    int64_t *offsets;             // [B + 1]
+    int32_t *region_rows;         // [B * regions] first packed row of every region (nullable)
+    unsigned long long *status;   // [1 + workgroups]: word 0 = error flag, then one word per workgroup
+};
+constexpr unsigned long long CHAIN_AGGREGATE = 1ull << 62, CHAIN_PREFIX = 2ull << 62;
+constexpr int CHAIN_SPIN_LIMIT = 1 << 20;
+
 // SCATTER = false: no packed rows at all - the kernel routes on `ref` as it stands and writes the records of its
 // rows (the first block of a model, which no scatter-back precedes); `in` then points, if anywhere, at `extra`
 // rows [extra, C] that are first copied into the extra-token rows of every sample of `out` (class / distillation
 // token plus their position embedding, the same for every sample).
-template <typename T, int GS, bool SUB, bool STAT = false, bool SCATTER = true>
-__global__ __launch_bounds__(256) void decompress_route_kernel(
+template <typename T, int GS, bool SUB, bool STAT = false, bool SCATTER = true, bool CHAIN = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CHAIN ? 4 : 1, CHAIN ? 4 : 8)))
+void decompress_route_kernel(
     const T *__restrict__ in, const T *__restrict__ sub, const int64_t *__restrict__ cur_indices,
     const int64_t *__restrict__ splits, const int64_t *__restrict__ offsets, const T *__restrict__ ref,
     T *__restrict__ out, const T *__restrict__ weight, const T *__restrict__ bias, T *__restrict__ gate,
     int64_t *__restrict__ indices, int B, int H, int W, int C, int extra, int S, int S2,
     u32x4 *__restrict__ records = nullptr, float eps = 0.f, const int64_t *__restrict__ next_splits = nullptr,
     uint8_t *__restrict__ next_counts = nullptr, const int32_t *__restrict__ region_rows = nullptr,
-    const uint8_t *__restrict__ cur_counts = nullptr)
+    const uint8_t *__restrict__ cur_counts = nullptr, const ChainArgs chain = ChainArgs{})
 {
     static_assert(!STAT || (GS == WAVE && std::is_same<T, bf16_t>::value), "records: one wave per region, bf16 rows");
+    static_assert(!CHAIN || (STAT && SCATTER), "the chained variant is the bf16 scatter-back with records");
     constexpr int VEC = Elem<T>::VEC;
     constexpr int R = 4;
     const int lane = threadIdx.x & (GS - 1);
@@ -1099,6 +1125,115 @@ __global__ __launch_bounds__(256) void decompress_route_kernel(
             const int ps2 = (int)next_splits[best_s];
             next_counts[region] = (uint8_t)(ps2 * ps2);
         }
+    }
+    if constexpr (CHAIN) {
+        // ---- the next block's packed rows of this region (the host launches whole workgroups of four regions)
+        __shared__ int cnt_s[4];
+        __shared__ long long excl_s;
+        const int wv = threadIdx.x >> 6;
+        const int ps_n = __builtin_amdgcn_readfirstlane((int)next_splits[best_s]);
+        const int nq = ps_n == 4 ? 16 : ps_n == 2 ? 4 : 1;
+        if (lane == 0) cnt_s[wv] = nq;
+        __syncthreads();
+        unsigned long long *st = chain.status + 1;
+        const int wg = (int)blockIdx.x;
+        if (wv == 0) {
+            const int agg = cnt_s[0] + cnt_s[1] + cnt_s[2] + cnt_s[3];
+            if (lane == 0)
+                __hip_atomic_store(st + wg, (wg == 0 ? CHAIN_PREFIX : CHAIN_AGGREGATE) | (unsigned long long)agg,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            long long excl = 0;
+            if (wg > 0) {
+                // Every step looks at LOOK x 64 words, nearest first.  One load a lane is the fastest: the nearest
+                // workgroups are the last to publish, and a wider window only makes each retry dearer (measured at
+                // 1024 workgroups: 52 us for the kernel with 64 words a step, 54 with 128, 57 with 512).
+                constexpr int LOOK = 1;
+                int j = wg - 1, spins = 0;
+                bool gave_up = false;
+                while (true) {
+                    unsigned long long v[LOOK];
+#pragma unroll
+                    for (int k = 0; k < LOOK; k++) {
+                        const int idx = j - lane - WAVE * k;   // lane 0 of k = 0: the workgroup just before this one
+                        v[k] = CHAIN_PREFIX;                   // before the first workgroup: a prefix of zero
+                        if (idx >= 0) v[k] = __hip_atomic_load(st + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    float part = 0.f;
+                    bool found = false, wait = false;
+#pragma unroll
+                    for (int k = 0; k < LOOK; k++) {
+                        if (!found && !wait) {
+                            const int flag = (int)(v[k] >> 62);
+                            const unsigned long long missing = __builtin_amdgcn_ballot_w64(flag == 0);
+                            const unsigned long long known = __builtin_amdgcn_ballot_w64(flag == 2);
+                            const int first_known = known ? __builtin_ctzll(known) : 64;
+                            const int first_missing = missing ? __builtin_ctzll(missing) : 64;
+                            if (first_missing < first_known) {
+                                wait = true;     // somebody nearer than the first prefix has not published yet
+                            } else {
+                                const int upto = first_known < 64 ? first_known : 63;
+                                part += lane <= upto ? (float)(unsigned)(v[k] & 0xffffffffull) : 0.f;
+                                found = first_known < 64;
+                            }
+                        }
+                    }
+                    if (wait) {
+                        if (++spins > CHAIN_SPIN_LIMIT) {
+                            gave_up = true;
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                        continue;
+                    }
+                    excl += (long long)wave_sum(part);
+                    if (found) break;
+                    j -= WAVE * LOOK;
+                }
+                if (gave_up) {
+                    excl = chain.capacity;                 // every row of this workgroup falls past the capacity
+                    if (lane == 0) __hip_atomic_store(chain.status, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (lane == 0)
+                    __hip_atomic_store(st + wg, CHAIN_PREFIX | (unsigned long long)(excl + agg), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (lane == 0) excl_s = excl;
+        }
+        __syncthreads();
+        long long rows_before = excl_s;
+        for (int w2 = 0; w2 < wv; w2++) rows_before += cnt_s[w2];
+        const int64_t n0 = rows_before + (int64_t)extra * (b + 1);        // first packed row of the region, next block
+        if (chain.region_rows != nullptr && lane == 0) chain.region_rows[region] = (int32_t)n0;
+        // descriptors, offsets (lengths are the differences of the offsets)
+        if (chain.patches != nullptr && lane < nq) {
+            const int pq = ps_n, step = R / pq;
+            const int dy = lane / pq, dx = lane - dy * pq;
+            const int64_t row = n0 + lane;
+            if (row >= 0 && row < chain.capacity) {
+                i64x2 *pp = reinterpret_cast<i64x2 *>(chain.patches + 4 * row);
+                pp[0] = i64x2{(long long)b, (long long)(ry * R + dy * step)};
+                pp[1] = i64x2{(long long)(rx * R + dx * step), (long long)step};
+            }
+        }
+        if (rr == 0) {
+            if (lane == 0) chain.offsets[b] = n0 - extra;
+            if (chain.patches != nullptr && lane < extra && n0 >= extra && n0 - extra + lane < chain.capacity) {
+                int64_t *pp = chain.patches + 4 * (n0 - extra + lane);
+                pp[0] = b; pp[1] = -(int64_t)lane - 1; pp[2] = 0; pp[3] = 1;
+            }
+        }
+        if (region == (int64_t)B * nreg - 1 && lane == 0) chain.offsets[B] = n0 + nq;
+        if (n0 < extra || n0 + nq > chain.capacity) return;   // never outside the buffers
+        // The tokens are read back by the lanes that stored them (a lane reads what it wrote itself, in program
+        // order): plain loads, served by the caches the stores went through.
+        const bool act = lane < nvec;
+        const int v = act ? lane : 0;
+        const bf16_t *xs = out + (int64_t)b * N * C + v * 8;
+        if (rr == 0)
+            pack_front_rows<bf16_t, true>(xs, chain.comp + (n0 - extra) * (int64_t)C + v * 8,
+                                          chain.comp_records + (n0 - extra) * 2, extra, C, chain.comp_eps, act, lane);
+        pack_region<bf16_t, true>(xs + tok0 * C, chain.comp + n0 * (int64_t)C + v * 8, chain.comp_records + n0 * 2,
+                                  ps_n, W, C, chain.comp_eps, act, lane);
     }
 }
 
@@ -1497,13 +1632,24 @@ extern "C" int vtdge_decompress_layernorm(const void *in, const void *sub, const
     return check_launch("decompress_layernorm");
 }
 
-extern "C" int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices,
-                                       const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
-                                       const void *next_weight, const void *next_bias, void *next_gate,
-                                       int64_t *next_indices, void *out_records, float records_eps,
-                                       const int64_t *next_splits, uint8_t *next_counts, const int32_t *region_rows,
-                                       const uint8_t *cur_counts, int B, int H, int W, int C, int extra, int R, int S,
-                                       int S2, int dtype, void *stream)
+namespace vtdge {
+
+// words of 64 bits the chained scatter-back needs for `regions` regions: the error word + one per workgroup
+static inline int64_t chain_words(int64_t regions) { return 1 + ceil_div(regions, (int64_t)ROWS_PER_BLOCK); }
+
+__global__ void clear_words_kernel(unsigned long long *p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}
+
+static int decompress_router_launch(const void *in, const void *sub, const int64_t *cur_indices,
+                                    const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
+                                    const void *next_weight, const void *next_bias, void *next_gate,
+                                    int64_t *next_indices, void *out_records, float records_eps,
+                                    const int64_t *next_splits, uint8_t *next_counts, const int32_t *region_rows,
+                                    const uint8_t *cur_counts, const ChainArgs *chain, int B, int H, int W, int C,
+                                    int extra, int R, int S, int S2, int dtype, void *stream)
 {
     VT_REQUIRE((region_rows == nullptr) == (cur_counts == nullptr), VTDGE_ERR_ARG,
                "decompress_router: the regions' first rows and their query counts come together");
@@ -1529,6 +1675,25 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
         VT_REQUIRE(dtype == VTDGE_BF16 && gs == WAVE && C / 8 <= WAVE, VTDGE_ERR_UNSUPPORTED,
                    "decompress_router: statistics records are written for bf16 rows of 264 to 512 channels (C=%d)", C);
         VT_REQUIRE(aligned16(out_records), VTDGE_ERR_ARG, "decompress_router: records must be 16-byte aligned");
+        if (chain != nullptr) {
+            // four regions to a workgroup, all present: the workgroups hand their query counts along
+            VT_REQUIRE(regions % ROWS_PER_BLOCK == 0 && regions <= 65536 &&
+                           (int64_t)B * (extra + (int64_t)H * W) < (1 << 24) && extra <= WAVE,
+                       VTDGE_ERR_UNSUPPORTED,
+                       "decompress_router_compress: %lld regions (a multiple of %d up to 65536), %d extra tokens (up to %d)",
+                       (long long)regions, ROWS_PER_BLOCK, extra, WAVE);
+            VT_REQUIRE(next_weight && next_splits && next_counts, VTDGE_ERR_ARG,
+                       "decompress_router_compress: needs the next router, its splits and the count bytes");
+#define VT_CHAIN(SUBF)                                                                                               \
+    note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<bf16_t, WAVE, SUBF, true, true, true>)),      \
+    decompress_route_kernel<bf16_t, WAVE, SUBF, true, true, true><<<grid, block, 0, st>>>(                           \
+        (const bf16_t *)in, (const bf16_t *)sub, cur_indices, splits, offsets, (const bf16_t *)ref, (bf16_t *)out,   \
+        (const bf16_t *)next_weight, (const bf16_t *)next_bias, (bf16_t *)next_gate, next_indices, B, H, W, C, extra, \
+        S, S2, (u32x4 *)out_records, records_eps, next_splits, next_counts, region_rows, cur_counts, *chain)
+            if (sub) VT_CHAIN(true); else VT_CHAIN(false);
+#undef VT_CHAIN
+            return check_launch("decompress_router_compress");
+        }
 #define VT_STAT(SUBF)                                                                                                \
     note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<bf16_t, WAVE, SUBF, true>)),                  \
     decompress_route_kernel<bf16_t, WAVE, SUBF, true><<<grid, block, 0, st>>>(                                       \
@@ -1554,6 +1719,67 @@ extern "C" int vtdge_decompress_router(const void *in, const void *sub, const in
 #undef VT_LAUNCH
 #undef VT_LAUNCH2
     return check_launch("decompress_router");
+}
+
+}  // namespace vtdge
+
+extern "C" int vtdge_decompress_router(const void *in, const void *sub, const int64_t *cur_indices,
+                                       const int64_t *splits, const int64_t *offsets, const void *ref, void *out,
+                                       const void *next_weight, const void *next_bias, void *next_gate,
+                                       int64_t *next_indices, void *out_records, float records_eps,
+                                       const int64_t *next_splits, uint8_t *next_counts, const int32_t *region_rows,
+                                       const uint8_t *cur_counts, int B, int H, int W, int C, int extra, int R, int S,
+                                       int S2, int dtype, void *stream)
+{
+    return decompress_router_launch(in, sub, cur_indices, splits, offsets, ref, out, next_weight, next_bias, next_gate,
+                                    next_indices, out_records, records_eps, next_splits, next_counts, region_rows,
+                                    cur_counts, nullptr, B, H, W, C, extra, R, S, S2, dtype, stream);
+}
+
+extern "C" int64_t vtdge_decompress_router_compress_workspace(int B, int H, int W, int R)
+{
+    if (B <= 0 || H <= 0 || W <= 0 || R <= 0) return 0;
+    return 8 * chain_words((int64_t)B * (H / R) * (W / R));
+}
+
+extern "C" int vtdge_decompress_router_compress(
+    const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits, const int64_t *offsets,
+    const void *ref, void *out, const void *next_weight, const void *next_bias, void *next_gate,
+    int64_t *next_indices, void *out_records, float records_eps, const int64_t *next_splits, uint8_t *next_counts,
+    const int32_t *region_rows, const uint8_t *cur_counts, void *next_comp, void *next_comp_records,
+    float next_records_eps, int64_t *next_patches, int64_t capacity_rows, int64_t *next_offsets,
+    int32_t *next_region_rows, void *workspace, int64_t workspace_bytes, int clear_workspace, int B, int H, int W,
+    int C, int extra, int R, int S, int S2, int dtype, void *stream)
+{
+    VT_REQUIRE(next_comp && next_comp_records && next_offsets && workspace && out_records, VTDGE_ERR_ARG,
+               "decompress_router_compress: NULL operand");
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && R == 4 && capacity_rows >= 0, VTDGE_ERR_ARG,
+               "decompress_router_compress: bad sizes");
+    VT_REQUIRE(dtype == VTDGE_BF16, VTDGE_ERR_UNSUPPORTED, "decompress_router_compress: bf16 rows only");
+    const int64_t words = chain_words((int64_t)B * (H / R) * (W / R));
+    VT_REQUIRE(workspace_bytes >= 8 * words && (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, VTDGE_ERR_ARG,
+               "decompress_router_compress: the workspace holds %lld bytes, %lld needed (8-byte aligned)",
+               (long long)workspace_bytes, (long long)(8 * words));
+    VT_REQUIRE(aligned16(next_comp) && aligned16(next_comp_records) && aligned16(next_patches), VTDGE_ERR_ARG,
+               "decompress_router_compress: operands must be 16-byte aligned");
+    if (clear_workspace) {
+        note_kernel(reinterpret_cast<const void *>(clear_words_kernel));
+        clear_words_kernel<<<dim3((unsigned)ceil_div(words, (int64_t)256)), dim3(256), 0, (hipStream_t)stream>>>(
+            (unsigned long long *)workspace, words);
+        if (int rc = check_launch("decompress_router_compress")) return rc;
+    }
+    ChainArgs chain;
+    chain.comp = (bf16_t *)next_comp;
+    chain.comp_records = (u32x4 *)next_comp_records;
+    chain.comp_eps = next_records_eps;
+    chain.patches = next_patches;
+    chain.capacity = capacity_rows;
+    chain.offsets = next_offsets;
+    chain.region_rows = next_region_rows;
+    chain.status = (unsigned long long *)workspace;
+    return decompress_router_launch(in, sub, cur_indices, splits, offsets, ref, out, next_weight, next_bias, next_gate,
+                                    next_indices, out_records, records_eps, next_splits, next_counts, region_rows,
+                                    cur_counts, &chain, B, H, W, C, extra, R, S, S2, dtype, stream);
 }
 
 extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *weight, const void *bias, void *gate,

@@ -72,6 +72,10 @@ ROUTER_STATS = True
 # `vtdge_compress_regions` leaves every region's first packed row for the scatter-back of the same block, which then
 # needs no sum over the gate indices before it can start on its rows.
 REGION_ROWS = True
+# The scatter-back also packs the next block's queries (`vtdge_decompress_router_compress`): the wave that has just
+# written a region's tokens and routed it reads them back from L2 and writes the next block's packed rows, their
+# records, descriptors and offsets, so that `vtdge_compress_regions` runs for a model's first block only.
+PACK_NEXT = True
 
 
 def _side_stream(device, slot=0):
@@ -222,6 +226,12 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
             g, idx = ops.router(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R)
         else:
             idx = g.argmax(dim=-1)
+        packed = carry.get("packed") if routed is not None else None
+        if packed is not None:
+            # the previous block's scatter-back has packed this block's queries already
+            if REGION_ROWS:
+                placed["region_rows"], placed["cur_counts"] = packed["region_rows"], carry["counts"]
+            return g, idx, packed["patches"], packed["offsets"], None, packed["comp"], None, packed["records"]
         if use_regions:
             # index->patch and compress in one kernel, by region; with the folded norm1 -> q it leaves the statistics
             # records of the packed rows instead of their normalised copy
@@ -312,6 +322,15 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         want_stats = (FOLD_NORMS and getattr(nattn, "sr_ratio", 1) <= 1 and ops.fits_scatter_stats(x)
                       and ops.fits_linear_layernorm(x, nattn.kv.weight))
         want_counts = REGION_COMPRESS and ops.fits_compress_regions(x, H, W, 4, nxt.router.split_sizes)
+        # the next block's queries too, where that block takes them with their records (norm1 folded into q) on one
+        # stream, as this one does
+        pack = (PACK_NEXT and want_stats and want_counts and fold1 and use_regions and not overlap
+                and ops.fits_pack_next(x, H, W, 4, nxt.router.split_sizes)
+                and ops.fits_linear_layernorm(x, nattn.q.weight))
+        spaces = carry.get("workspaces")
+        if pack:
+            placed.update(pack_next=True, pack_eps=next_block.norm1.eps, capacity=cap,
+                          workspace=spaces.pop() if spaces else None)
         res = ops.decompress_router(q2, indices, dge.splits, offsets, x, H, W, R, sub=comp,
                                     next_weight=nxt.router.gate.weight, next_bias=nxt.router.gate.bias,
                                     stats_eps=next_block.norm1.eps if want_stats else None,
@@ -321,21 +340,34 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         if want_stats:
             handed["x_stats"] = res[3]
         if want_counts:
-            handed["counts"] = res[-1]
+            handed["counts"] = res[4 if want_stats else 3]
+        if pack:
+            handed["packed"] = res[5]
+        if spaces:
+            handed["workspaces"] = spaces
     else:
         out = ops.decompress(q2, patches, x, W, extra, add_ref=True, sub=comp, rows_dev=rows_dev, rows=cap)
 
     # `states` as the reference's code reads it (vtpack/layers/dge.py:81-84): the host-side counts and the tensors cut
     # to the live rows are produced when they are read (one device->host copy per read, nothing cached: a graph replay
     # rewrites `lengths` without running this code); nothing is copied otherwise.
+    came_packed = carry.get("packed") if lengths is None else None
+
+    def live():
+        if came_packed is not None and int(came_packed["workspace"][0]) != 0:
+            raise RuntimeError("the scatter-back that packed this block's queries gave up waiting (see "
+                               "vtdge_decompress_router_compress): rows are missing")
+        return offsets[1:] - offsets[:-1] if lengths is None else lengths
+
     def batches():
-        return lengths.cpu()
+        return live().cpu()
 
     def cut(t):
-        return lambda: t[:int(lengths.sum())]
+        return lambda: t[:int(live().sum())]
 
     dge.states.update({"comp": Deferred(cut(comp)), "input": x, "patches": Deferred(cut(patches)),
-                       "batches": Deferred(batches), "batches_device": lengths, "offsets_device": offsets,
+                       "batches": Deferred(batches),
+                       "batches_device": Deferred(live) if lengths is None else lengths, "offsets_device": offsets,
                        "gate": gate, "size": (H, W), "num_extra_tokens": extra, "queries": Deferred(cut(q2))})
     if next_block is not None:
         return out, handed
@@ -345,7 +377,13 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
 def _run_blocks(blocks, x, H, W, front=None):
     """A chain of blocks on one token grid, each handing the next what it has already computed for it.  `front`
     [extra, C]: rows the first block stores as the extra tokens of every sample before anything reads them."""
-    carry = {"front": front} if front is not None else None
+    carry = {"front": front} if front is not None else {}
+    R = blocks[0].dge.region_size if blocks else 0
+    if (PACK_NEXT and len(blocks) > 1 and R == 4
+            and ops.fits_pack_next(x, H, W, R, blocks[0].dge.router.split_sizes)):
+        # one zeroed slice of workspace per scatter-back that packs the next block's queries, cleared in one go
+        words = ops.pack_next_workspace_words(x.shape[0], H, W, R)
+        carry["workspaces"] = list(torch.zeros((len(blocks) - 1, words), dtype=torch.int64, device=x.device).unbind(0))
     for i, blk in enumerate(blocks):
         if i + 1 < len(blocks):
             x, carry = block_forward(blk, x, H, W, carry=carry, next_block=blocks[i + 1])

@@ -235,9 +235,22 @@ def compress_regions(x, indices, splits, H, W, region_size=4, counts=None, stats
     return comp, rec, patches, offsets, lengths
 
 
+def pack_next_workspace_words(B, H, W, region_size=4):
+    """64-bit words of workspace `decompress_router(..., pack_next=True)` needs."""
+    return int(_lib.load().vtdge_decompress_router_compress_workspace(B, H, W, region_size)) // 8
+
+
+def fits_pack_next(x, H, W, region_size, split_sizes):
+    """True when `decompress_router(..., pack_next=True)` takes these tokens: what `compress_regions` and the
+    statistics records need, and whole workgroups of four regions."""
+    B = x.shape[0]
+    return (fits_compress_regions(x, H, W, region_size, split_sizes) and fits_scatter_stats(x)
+            and (B * (H // region_size) * (W // region_size)) % 4 == 0)
+
+
 def decompress_router(inp, indices, splits, offsets, reference, H, W, region_size, sub=None, next_weight=None,
                       next_bias=None, want_gate=True, stats_eps=None, next_splits=None, region_rows=None,
-                      cur_counts=None):
+                      cur_counts=None, pack_next=False, pack_eps=None, capacity=None, workspace=None):
     """Scatter (inp - sub) + reference back over the tokens by region, and route the NEXT block on the result:
     -> (out, next_gate or None, next_indices or None), and with `stats_eps` (a LayerNorm's eps; bf16 rows of 264 to
     512 channels) a fourth value: the statistics records of the rows of `out` for `linear_layernorm`; with `next_splits`
@@ -245,7 +258,14 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
     regions for `compress_regions`.  `indices` [B, Hr, Wr] are this block's gate indices, `offsets` [B+1] the prefix of
     its query counts; `region_rows` with `cur_counts` (from this block's `compress_regions` and the count bytes it
     read) spare the kernel adding a region's place up from them.  The three outputs equal decompress(...) and router(out, next_weight,
-    next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75."""
+    next_bias) bit for bit.  vtpack/layers/dge.py:87-112 and, for the next block, :145-150, :75.
+
+    `pack_next` (see `fits_pack_next`; needs stats_eps and next_splits): the kernel also packs the next block's
+    queries, as `compress_regions(out, next_indices, next_splits, counts=...)` would, and the result ends with a dict
+    of comp [capacity, C], records (LayerNorm eps `pack_eps`), patches, offsets [B+1], region_rows and `workspace`,
+    whose first word stays 0 unless the kernel failed.  `workspace` is a zeroed int64 tensor of
+    `pack_next_workspace_words(...)` words that nothing else uses meanwhile; without it the call makes and clears
+    one."""
     _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
     inp, reference = _contig(inp), _contig(reference)
     sub = None if sub is None else _contig(sub)
@@ -291,6 +311,36 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
             raise ValueError("region_rows must be int32 with one entry per region, cur_counts the uint8 buffer beside it")
     if next_splits is not None:
         counts = region_counts_buffer(B, (H // region_size) * (W // region_size), inp.device)
+    if pack_next:
+        if rec is None or counts is None or pack_eps is None:
+            raise ValueError("pack_next needs stats_eps, next_splits and pack_eps")
+        regions = B * (H // region_size) * (W // region_size)
+        if capacity is None:
+            capacity = B * N
+        if capacity < B * N:
+            raise ValueError("the packed rows are written without bounds checks: capacity must be at least B * N")
+        words = pack_next_workspace_words(B, H, W, region_size)
+        clear = workspace is None
+        if clear:
+            workspace = torch.empty((words,), dtype=torch.int64, device=inp.device)
+        elif workspace.dtype != torch.int64 or workspace.numel() < words or not workspace.is_contiguous():
+            raise ValueError(f"workspace must be a contiguous int64 tensor of at least {words} words")
+        ncomp = torch.empty((capacity, C), dtype=inp.dtype, device=inp.device)
+        nrec = torch.empty((capacity, 16), dtype=torch.bfloat16, device=inp.device)
+        npat = torch.empty((capacity, 4), dtype=torch.int64, device=inp.device)
+        noff = torch.empty((B + 1,), dtype=torch.int64, device=inp.device)
+        nrows = torch.empty((regions,), dtype=torch.int32, device=inp.device)
+        head = (ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference), ptr(out),
+                ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), ptr(rec), float(stats_eps), ptr(next_splits),
+                ptr(counts), ptr(region_rows), ptr(cur_counts), ptr(ncomp), ptr(nrec), float(pack_eps), ptr(npat),
+                capacity, ptr(noff), ptr(nrows))
+        tail = (B, H, W, C, extra, region_size, S, S2, dtype_code(inp), stream_ptr())
+        _need_gpu(workspace)
+        call("vtdge_decompress_router_compress", *head, ptr(workspace), workspace.numel() * 8, int(clear), *tail,
+             tag=("decompress_router_compress", sub is not None, C, True))
+        packed = {"comp": ncomp, "records": nrec, "patches": npat, "offsets": noff, "region_rows": nrows,
+                  "workspace": workspace}
+        return (out, gate, nidx, rec, counts, packed)
     call("vtdge_decompress_router", ptr(inp), ptr(sub), ptr(indices), ptr(splits), ptr(offsets), ptr(reference),
          ptr(out), ptr(next_weight), ptr(next_bias), ptr(gate), ptr(nidx), ptr(rec),
          float(stats_eps if stats_eps is not None else 0.0), ptr(next_splits), ptr(counts), ptr(region_rows),
