@@ -180,6 +180,26 @@ int vtdge_decompress_router_compress(const void *in, const void *sub, const int6
                                      int64_t workspace_bytes, int clear_workspace, int B, int H, int W, int C,
                                      int extra, int R, int S, int S2, int dtype, void *stream);
 
+/* vtdge_decompress_router_compress for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc); it has no counterpart in the reference.  The arguments are
+ * those of vtdge_decompress_router_compress without the workspace: the status words live in an array inside the
+ * library's device image (128 KB on every GPU the library runs on, held until the process ends), cleared by a small
+ * fill kernel on `stream` before the kernel runs.  The call allocates and frees nothing.  At most 65536 regions
+ * (VTDGE_ERR_UNSUPPORTED beyond).  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * two threads) race - run them in turn.  The first call on a GPU looks the array's address up
+ * (hipGetSymbolAddress) and should therefore come before any stream capture.  A kernel that gave up shows as
+ * next_offsets[B] > capacity_rows, as in vtdge_decompress_router_compress. */
+int vtdge_decompress_router_compress_static(const void *in, const void *sub, const int64_t *cur_indices,
+                                            const int64_t *splits, const int64_t *offsets, const void *ref,
+                                            void *out, const void *next_weight, const void *next_bias,
+                                            void *next_gate, int64_t *next_indices, void *out_records,
+                                            float records_eps, const int64_t *next_splits, uint8_t *next_counts,
+                                            const int32_t *region_rows, const uint8_t *cur_counts, void *next_comp,
+                                            void *next_comp_records, float next_records_eps, int64_t *next_patches,
+                                            int64_t capacity_rows, int64_t *next_offsets, int32_t *next_region_rows,
+                                            int B, int H, int W, int C, int extra, int R, int S, int S2, int dtype,
+                                            void *stream);
+
 /* The router of a model's FIRST block together with the statistics records of all its tokens (no scatter-back
  * precedes it that could leave them): vtdge_router and vtdge_layernorm_stats in one pass over x, i.e.
  * DynamicRouter.forward + argmax (vtpack/layers/dge.py:145-150, :75) and the statistics half of norm1

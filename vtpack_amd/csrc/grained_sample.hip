@@ -8,6 +8,7 @@
 // first PVT stages) still keep every lane of the wavefront busy.
 #include "common.h"
 #include "region_pack.h"
+#include <atomic>
 #include <type_traits>
 
 namespace vtdge {
@@ -1740,6 +1741,48 @@ extern "C" int64_t vtdge_decompress_router_compress_workspace(int B, int H, int 
 {
     if (B <= 0 || H <= 0 || W <= 0 || R <= 0) return 0;
     return 8 * chain_words((int64_t)B * (H / R) * (W / R));
+}
+
+// ---- the same call for callers that cannot allocate device memory: the status words live in the library's image
+namespace vtdge {
+constexpr int64_t STATIC_CHAIN_REGIONS = 65536;      // the kernel's own limit
+constexpr int64_t STATIC_CHAIN_WORDS = 1 + STATIC_CHAIN_REGIONS / ROWS_PER_BLOCK;
+static __device__ __align__(256) unsigned long long scratch[STATIC_CHAIN_WORDS];     // 128 KB + 8 bytes per GPU
+constexpr int MAX_DEVICES = 64;
+static std::atomic<unsigned long long *> scratch_ptr[MAX_DEVICES];     // the array's address on every GPU seen so far
+}  // namespace vtdge
+
+extern "C" int vtdge_decompress_router_compress_static(
+    const void *in, const void *sub, const int64_t *cur_indices, const int64_t *splits, const int64_t *offsets,
+    const void *ref, void *out, const void *next_weight, const void *next_bias, void *next_gate,
+    int64_t *next_indices, void *out_records, float records_eps, const int64_t *next_splits, uint8_t *next_counts,
+    const int32_t *region_rows, const uint8_t *cur_counts, void *next_comp, void *next_comp_records,
+    float next_records_eps, int64_t *next_patches, int64_t capacity_rows, int64_t *next_offsets,
+    int32_t *next_region_rows, int B, int H, int W, int C, int extra, int R, int S, int S2, int dtype, void *stream)
+{
+    VT_REQUIRE(B > 0 && H > 0 && W > 0 && R == 4, VTDGE_ERR_ARG, "decompress_router_compress_static: bad sizes");
+    const int64_t regions = (int64_t)B * (H / R) * (W / R);
+    VT_REQUIRE(regions <= STATIC_CHAIN_REGIONS, VTDGE_ERR_UNSUPPORTED,
+               "decompress_router_compress_static: %lld regions, the built-in workspace holds %lld", (long long)regions,
+               (long long)STATIC_CHAIN_REGIONS);
+    int dev = -1;
+    VT_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES, VTDGE_ERR_LAUNCH,
+               "decompress_router_compress_static: no current device (or more than %d)", MAX_DEVICES);
+    unsigned long long *ws = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ws == nullptr) {
+        // every GPU holds its own copy of the array at its own address: ask for it once, with that GPU current
+        const hipError_t rc = hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(scratch));
+        VT_REQUIRE(rc == hipSuccess && ws != nullptr, VTDGE_ERR_LAUNCH,
+                   "decompress_router_compress_static: hipGetSymbolAddress: %s", hipGetErrorString(rc));
+        scratch_ptr[dev].store(ws, std::memory_order_release);
+    }
+    // the words of this call start at zero (a fill kernel, not a memset: the call may be under stream capture)
+    return vtdge_decompress_router_compress(in, sub, cur_indices, splits, offsets, ref, out, next_weight, next_bias,
+                                            next_gate, next_indices, out_records, records_eps, next_splits,
+                                            next_counts, region_rows, cur_counts, next_comp, next_comp_records,
+                                            next_records_eps, next_patches, capacity_rows, next_offsets,
+                                            next_region_rows, ws, 8 * STATIC_CHAIN_WORDS, 1, B, H, W, C, extra, R, S,
+                                            S2, dtype, stream);
 }
 
 extern "C" int vtdge_decompress_router_compress(

@@ -265,7 +265,8 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
     of comp [capacity, C], records (LayerNorm eps `pack_eps`), patches, offsets [B+1], region_rows and `workspace`,
     whose first word stays 0 unless the kernel failed.  `workspace` is a zeroed int64 tensor of
     `pack_next_workspace_words(...)` words that nothing else uses meanwhile; without it the call makes and clears
-    one."""
+    one; "static" takes the array built into the library (`vtdge_decompress_router_compress_static`: no allocation
+    inside the library call, one call at a time per GPU), and the dict's `workspace` is then None."""
     _need_gpu(inp, indices, splits, offsets, reference, sub, next_weight, next_bias)
     inp, reference = _contig(inp), _contig(reference)
     sub = None if sub is None else _contig(sub)
@@ -320,8 +321,11 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
         if capacity < B * N:
             raise ValueError("the packed rows are written without bounds checks: capacity must be at least B * N")
         words = pack_next_workspace_words(B, H, W, region_size)
+        built_in = isinstance(workspace, str) and workspace == "static"
         clear = workspace is None
-        if clear:
+        if built_in:
+            workspace = None
+        elif clear:
             workspace = torch.empty((words,), dtype=torch.int64, device=inp.device)
         elif workspace.dtype != torch.int64 or workspace.numel() < words or not workspace.is_contiguous():
             raise ValueError(f"workspace must be a contiguous int64 tensor of at least {words} words")
@@ -335,9 +339,13 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
                 ptr(counts), ptr(region_rows), ptr(cur_counts), ptr(ncomp), ptr(nrec), float(pack_eps), ptr(npat),
                 capacity, ptr(noff), ptr(nrows))
         tail = (B, H, W, C, extra, region_size, S, S2, dtype_code(inp), stream_ptr())
-        _need_gpu(workspace)
-        call("vtdge_decompress_router_compress", *head, ptr(workspace), workspace.numel() * 8, int(clear), *tail,
-             tag=("decompress_router_compress", sub is not None, C, True))
+        if built_in:       # the status words inside the library: the call itself allocates nothing
+            call("vtdge_decompress_router_compress_static", *head, *tail,
+                 tag=("decompress_router_compress", sub is not None, C, True))
+        else:
+            _need_gpu(workspace)
+            call("vtdge_decompress_router_compress", *head, ptr(workspace), workspace.numel() * 8, int(clear), *tail,
+                 tag=("decompress_router_compress", sub is not None, C, True))
         packed = {"comp": ncomp, "records": nrec, "patches": npat, "offsets": noff, "region_rows": nrows,
                   "workspace": workspace}
         return (out, gate, nidx, rec, counts, packed)
