@@ -1028,6 +1028,7 @@ void decompress_route_kernel(
     // STAT: the host sends rows of at most GS vectors, and every lane makes the one trip (lanes past the row idle
     // inside it, present for the sums over the wave)
     const int vend = STAT ? GS : nvec;
+    u32x4 pooled = {0u, 0u, 0u, 0u};      // CHAIN: this lane's vector of the region's mean as the router rounds it
     for (int v0 = lane; v0 < vend; v0 += GS) {
         const bool act = !STAT || v0 < nvec;
         const int v = act ? v0 : 0;
@@ -1094,6 +1095,7 @@ void decompress_route_kernel(
         if (weight != nullptr && act) {
 #pragma unroll
             for (int i = 0; i < VEC; i++) acc[i] = Elem<T>::round(acc[i] / (float)(R * R));
+            if constexpr (CHAIN) pooled = Elem<T>::pack(acc);
 #pragma unroll
             for (int s = 0; s < VTDGE_MAX_SPLITS; s++) {
                 if (s < S2) {
@@ -1233,8 +1235,20 @@ void decompress_route_kernel(
         if (rr == 0)
             pack_front_rows<bf16_t, true>(xs, chain.comp + (n0 - extra) * (int64_t)C + v * 8,
                                           chain.comp_records + (n0 - extra) * 2, extra, C, chain.comp_eps, act, lane);
-        pack_region<bf16_t, true>(xs + tok0 * C, chain.comp + n0 * (int64_t)C + v * 8, chain.comp_records + n0 * 2,
-                                  ps_n, W, C, chain.comp_eps, act, lane);
+        if (ps_n == 1) {
+            // one query for the whole region: the mean of its 16 tokens, which the router has just taken (the same
+            // sum in the same order, the same single rounding) - nothing to read back
+            if (act) *reinterpret_cast<u32x4 *>(chain.comp + n0 * (int64_t)C + v * 8) = pooled;
+            float pivot, sums[2];
+            lane_sums<bf16_t>(pooled, act, pivot, sums[0], sums[1]);
+            wave_sum_n<2>(sums);
+            u32x4 lo, hi;
+            row_record(pivot, sums[0], sums[1], C, chain.comp_eps, lo, hi);
+            if (lane < 2) chain.comp_records[n0 * 2 + lane] = lane ? hi : lo;
+        } else {
+            pack_region<bf16_t, true>(xs + tok0 * C, chain.comp + n0 * (int64_t)C + v * 8,
+                                      chain.comp_records + n0 * 2, ps_n, W, C, chain.comp_eps, act, lane);
+        }
     }
 }
 
