@@ -210,10 +210,13 @@ int vtdge_decompress_router_compress_static(const void *in, const void *sub, con
  *   front_rows (nullable) [extra, C]: rows that are first stored as tokens 0 .. extra-1 of EVERY sample of x - the
  *   class (and distillation) token plus its position embedding, which the reference concatenates in front of the
  *   patch tokens (deit_dge.py:270-277) and which do not depend on the sample.
+ *   clear_words (nullable) with n_clear_words: 64-bit words the launch sets to zero on the way - the workspaces of
+ *   the vtdge_decompress_router_compress calls that follow it on the stream, so that a forward needs no fill kernel.
  * bf16 rows of 264 to 512 channels, R = 4. */
 int vtdge_router_stats(void *x, const void *front_rows, const void *weight, const void *bias, void *gate,
                        int64_t *indices, void *records, float records_eps, const int64_t *splits, uint8_t *counts,
-                       int B, int H, int W, int C, int extra, int R, int S, int dtype, void *stream);
+                       void *clear_words, int64_t n_clear_words, int B, int H, int W, int C, int extra, int R, int S,
+                       int dtype, void *stream);
 
 /* Gate indices -> packed queries in one step, by region: vtdge_index_to_patch and vtdge_compress together, i.e.
  * grained_sample_index_to_patch followed by grained_sample_compress

@@ -339,8 +339,11 @@ def test_router_with_records_of_all_tokens(dev, B, H, Cc, extra, with_front):
     assert_record_layout(rec)
     assert float((mean.double() - m_ref).abs().max()) < 5e-6 * float(want_x.double().abs().max())
     assert float(((sigma.double() - s_ref) / s_ref).abs().max()) < 3e-5
-    _, _, rec2, none = ops.router_stats(x, wgt, bias, H, W, 4, EPS)
+    # words to clear on the way (more of them than the launch has threads at the small shapes)
+    scratch = torch.full((5001,), -1, dtype=torch.int64, device=dev)
+    _, _, rec2, none = ops.router_stats(x, wgt, bias, H, W, 4, EPS, clear=scratch[:5000])
     assert none is None and torch.equal(rec2, rec)
+    assert int(scratch[:5000].abs().sum()) == 0 and int(scratch[5000]) == -1
 
 
 def test_scatter_records_refused_for_other_rows(dev):

@@ -985,6 +985,13 @@ void decompress_route_kernel(
     constexpr int R = 4;
     const int lane = threadIdx.x & (GS - 1);
     const int Hr = H / R, Wr = W / R, nreg = Hr * Wr;
+    if constexpr (!SCATTER) {
+        // the first kernel of a forward also clears `chain.capacity` 64-bit words at `chain.status` (the status words
+        // of the chained scatter-backs that follow it on the stream)
+        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chain.capacity;
+             i += (int64_t)gridDim.x * blockDim.x)
+            chain.status[i] = 0ull;
+    }
     const int64_t region = ((int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6)) * (WAVE / GS) + (threadIdx.x & 63) / GS;
     if (region >= (int64_t)B * nreg) return;
     const int b = (int)(region / nreg);
@@ -1841,9 +1848,12 @@ extern "C" int vtdge_decompress_router_compress(
 
 extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *weight, const void *bias, void *gate,
                                   int64_t *indices, void *records, float records_eps, const int64_t *splits,
-                                  uint8_t *counts, int B, int H, int W, int C, int extra, int R, int S, int dtype,
-                                  void *stream)
+                                  uint8_t *counts, void *clear_words, int64_t n_clear_words, int B, int H, int W,
+                                  int C, int extra, int R, int S, int dtype, void *stream)
 {
+    VT_REQUIRE(n_clear_words >= 0 && (n_clear_words == 0 || clear_words != nullptr) &&
+                   (reinterpret_cast<uintptr_t>(clear_words) & 7u) == 0,
+               VTDGE_ERR_ARG, "router_stats: the words to clear need an 8-byte aligned pointer");
     VT_REQUIRE(x && weight && bias && indices && records, VTDGE_ERR_ARG, "router_stats: NULL operand");
     VT_REQUIRE(counts == nullptr || splits != nullptr, VTDGE_ERR_ARG, "router_stats: the query counts need the splits");
     VT_REQUIRE(B > 0 && H > 0 && W > 0 && extra >= 0, VTDGE_ERR_ARG, "router_stats: bad sizes");
@@ -1858,11 +1868,14 @@ extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *w
                "router_stats: operands must be 16-byte aligned");
     const int64_t regions = (int64_t)B * (H / R) * (W / R);
     dim3 grid((unsigned)ceil_div(regions, ROWS_PER_BLOCK)), block(256);
+    ChainArgs side = {};            // no packing here: only the words this launch clears on the way
+    side.status = (unsigned long long *)clear_words;
+    side.capacity = n_clear_words;
     note_kernel(reinterpret_cast<const void *>(decompress_route_kernel<bf16_t, WAVE, false, true, false>));
     decompress_route_kernel<bf16_t, WAVE, false, true, false><<<grid, block, 0, (hipStream_t)stream>>>(
         (const bf16_t *)front_rows, nullptr, nullptr, splits, nullptr, (const bf16_t *)x, (bf16_t *)x,
         (const bf16_t *)weight, (const bf16_t *)bias, (bf16_t *)gate, indices, B, H, W, C, extra, S, S,
-        (u32x4 *)records, records_eps, splits, counts);
+        (u32x4 *)records, records_eps, splits, counts, nullptr, nullptr, side);
     return check_launch("router_stats");
 }
 

@@ -188,11 +188,14 @@ def block_forward(block, x, H, W, gate=None, overlap=True, carry=None, next_bloc
         # a model's first block: its router, the statistics records of all tokens for norm1 -> kv, the query counts
         # of its regions and, on the way, the class-token rows put in front of every sample, in one pass over x
         g0, i0, rec0, cnt0 = ops.router_stats(x, dge.router.gate.weight, dge.router.gate.bias, H, W, R, n1.eps,
-                                              front_rows=front, splits=dge.splits if use_regions else None)
+                                              front_rows=front, splits=dge.splits if use_regions else None,
+                                              clear=carry.get("clear"))
         routed = (g0, i0)
-        carry = dict(carry, x_stats=rec0, counts=cnt0)
+        carry = dict(carry, x_stats=rec0, counts=cnt0, clear=None)
     elif front is not None:
         x[:, :front.shape[0], :] = front
+    if carry.get("clear") is not None:      # workspaces of the blocks' scatter-backs that no kernel has cleared yet
+        carry["clear"].zero_()
 
     fuse_rn = (FUSE_ROUTER_NORM and gate is None and routed is None and x_ln is None
                and ops.fits_router_layernorm(x, R))
@@ -381,9 +384,11 @@ def _run_blocks(blocks, x, H, W, front=None):
     R = blocks[0].dge.region_size if blocks else 0
     if (PACK_NEXT and len(blocks) > 1 and R == 4
             and ops.fits_pack_next(x, H, W, R, blocks[0].dge.router.split_sizes)):
-        # one zeroed slice of workspace per scatter-back that packs the next block's queries, cleared in one go
+        # one slice of workspace per scatter-back that packs the next block's queries, all cleared by the first
+        # block's first kernel
         words = ops.pack_next_workspace_words(x.shape[0], H, W, R)
-        carry["workspaces"] = list(torch.zeros((len(blocks) - 1, words), dtype=torch.int64, device=x.device).unbind(0))
+        spaces = torch.empty((len(blocks) - 1, words), dtype=torch.int64, device=x.device)
+        carry["workspaces"], carry["clear"] = list(spaces.unbind(0)), spaces
     for i, blk in enumerate(blocks):
         if i + 1 < len(blocks):
             x, carry = block_forward(blk, x, H, W, carry=carry, next_block=blocks[i + 1])

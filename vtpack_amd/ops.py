@@ -358,11 +358,13 @@ def decompress_router(inp, indices, splits, offsets, reference, H, W, region_siz
     return res
 
 
-def router_stats(x, weight, bias, H, W, region_size, stats_eps, front_rows=None, splits=None, want_gate=True):
+def router_stats(x, weight, bias, H, W, region_size, stats_eps, front_rows=None, splits=None, want_gate=True,
+                 clear=None):
     """`router` and `layernorm_stats` of every token in one pass over x [B, extra + H*W, C] (bf16, see
     `fits_scatter_stats`): -> (gate or None, indices, records [B*N, 16], counts or None).  `front_rows` [extra, C] are
     first written into the extra-token rows of every sample of x (in place); with `splits` (int64, device) the uint8
-    query counts per region are left for `compress_regions`."""
+    query counts per region are left for `compress_regions`.  `clear`: a contiguous int64 tensor the launch zeroes on
+    its way (the workspaces of the `decompress_router(..., pack_next=True)` calls that follow)."""
     _need_gpu(x, weight, bias, front_rows, splits)
     if not x.is_contiguous():
         raise ValueError("router_stats works on x in place: it must be contiguous")
@@ -386,8 +388,13 @@ def router_stats(x, weight, bias, H, W, region_size, stats_eps, front_rows=None,
             raise ValueError("splits must be int64 with one entry per row of the router's weight")
         splits = _contig(splits)
         counts = region_counts_buffer(B, Hr * Wr, x.device)
+    if clear is not None:
+        _need_gpu(clear)
+        if clear.dtype != torch.int64 or not clear.is_contiguous():
+            raise ValueError("clear must be a contiguous int64 tensor")
     call("vtdge_router_stats", ptr(x), ptr(front_rows), ptr(weight), ptr(bias), ptr(gate), ptr(indices), ptr(rec),
-         float(stats_eps), ptr(splits), ptr(counts), B, H, W, C, extra, region_size, S, dtype_code(x), stream_ptr(),
+         float(stats_eps), ptr(splits), ptr(counts), ptr(clear), clear.numel() if clear is not None else 0,
+         B, H, W, C, extra, region_size, S, dtype_code(x), stream_ptr(),
          tag=("router_stats", C))
     return gate, indices, rec, counts
 
