@@ -366,7 +366,9 @@ def test_scatter_records_refused_for_other_rows(dev):
 @pytest.mark.parametrize("B,H,W,Cc,extra,with_sub", [(8, 16, 16, 384, 1, True), (4, 32, 32, 384, 2, True),
                                                      (4, 8, 8, 512, 0, False), (2, 8, 8, 264, 1, True),
                                                      (3, 8, 16, 384, 1, True), (256, 16, 16, 384, 1, True),
-                                                     (64, 32, 32, 384, 0, True)])
+                                                     (64, 32, 32, 384, 0, True),
+                                                     # four times as many workgroups as the chip holds at once
+                                                     (256, 32, 32, 384, 1, True)])
 def test_scatter_back_packs_the_next_queries(dev, B, H, W, Cc, extra, with_sub):
     from vtpack_amd import ops
     N = extra + H * W
