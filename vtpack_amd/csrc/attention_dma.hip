@@ -122,24 +122,28 @@ __device__ __forceinline__ u32x4 att_scale_frag(const u32x4 &q, float f)
     r.w = pack_bf16x2(bf16lo(q.w) * f, bf16hi(q.w) * f);
     return r;
 }
-// The largest of a lane's 16 scores in eight instructions: v_max3_f32 written out, because fmaxf() on values whose
-// origin the compiler cannot see (the output of an MFMA) comes with one more instruction per operand that quiets
-// signalling NaNs (14 instructions for the same maximum, a quarter of the softmax's full-rate vector work).
-__device__ __forceinline__ float att_max3(float a, float b, float c)
-{
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
 __device__ __forceinline__ float att_max16(const f32x16 &s)
 {
-    float a = att_max3(s[0], s[1], s[2]), b = att_max3(s[8], s[9], s[10]);
-    a = att_max3(a, s[3], s[4]);
-    b = att_max3(b, s[11], s[12]);
-    a = att_max3(a, s[5], s[6]);
-    b = att_max3(b, s[13], s[14]);
-    a = att_max3(a, s[7], s[15]);
-    return att_max3(a, b, b);
+    const float a = fmaxf(fmaxf(fmaxf(s[0], s[1]), s[2]), fmaxf(fmaxf(s[3], s[4]), s[5]));
+    const float b = fmaxf(fmaxf(fmaxf(s[6], s[7]), s[8]), fmaxf(fmaxf(s[9], s[10]), s[11]));
+    return fmaxf(fmaxf(a, b), fmaxf(fmaxf(fmaxf(s[12], s[13]), s[14]), s[15]));
+}
+// The largest of a lane's 16 scores IF one of them is positive (else some negative value): the maximum of their bit
+// patterns as signed integers, which orders positive floats as floats and puts every negative one below them.  That
+// is all the test against the (positive) rescaling threshold needs, and it takes eight v_max3_i32, where fmaxf() on
+// values whose origin the compiler cannot see (the output of an MFMA) brings one more instruction per operand to
+// quiet signalling NaNs: 14 instructions for the same decision, a quarter of the softmax's full-rate vector work.
+__device__ __forceinline__ float att_max16_if_positive(const f32x16 &s)
+{
+    const auto bits = [&](int e) { return __float_as_int(s[e]); };
+    const auto max3 = [](int a, int b, int c) { return max(max(a, b), c); };
+    int a = max3(bits(0), bits(1), bits(2)), b = max3(bits(8), bits(9), bits(10));
+    a = max3(a, bits(3), bits(4));
+    b = max3(b, bits(11), bits(12));
+    a = max3(a, bits(5), bits(6));
+    b = max3(b, bits(13), bits(14));
+    a = max3(a, bits(7), bits(15));
+    return __int_as_float(max(a, b));
 }
 
 // One step of the pipeline: softmax of block kb (scores relative to the reference in `sc`) and O^T += V^T P^T,
@@ -159,7 +163,7 @@ __device__ __forceinline__ void att_step(const AttnTile &t, const int (&cs)[4], 
         for (int e = 0; e < 16; e++)
             if (8 * (e >> 2) + (e & 3) >= lim) sc[e] = -INFINITY;
     }
-    const float mx = att_max16(sc);
+    const float mx = att_max16_if_positive(sc);
     if (__builtin_amdgcn_ballot_w64(mx > ATT_RESCALE) != 0) {      // wave-uniform and rare
         const float mrow = fmaxf(mx, __shfl_xor(mx, 32, WAVE));     // both lanes of a row decide alike
         const float delta = mrow > ATT_RESCALE ? mrow : 0.f;
