@@ -60,6 +60,8 @@ __device__ __forceinline__ float bf16_pair_sum(uint32_t pair, float acc)
 struct AttnTile {
     const unsigned char *krow;      // K row `lr` of block 0 in LDS
     const unsigned char *vlane;     // this lane's source address for the transposing reads of V, block 0, d < 32
+    const unsigned char *vlane_hi;  // HI: the same for d >= 32, vlane ^ 64 (key offsets are multiples of 128 bytes,
+                                    // so the XOR can be taken once and every read is a base plus a constant)
     int n, lg;
 };
 
@@ -91,6 +93,9 @@ __device__ __forceinline__ const unsigned char *att_v_lane(const unsigned char *
     const int chunk = (2 * (blk & 1) + (r >> 1)) ^ (2 * (key & 3));
     return vbase + key * 128 + chunk * 16 + 8 * (r & 1);
 }
+// HI: the tile carries the address for d >= 32 (two instructions a block less; in the resident kernel the extra
+// register costs more than they do: 45 against 38 us)
+template <bool HI>
 __device__ __forceinline__ void att_read_v(const AttnTile &t, int kb, u32x4 (&vf)[4])
 {
 #pragma unroll
@@ -98,7 +103,8 @@ __device__ __forceinline__ void att_read_v(const AttnTile &t, int kb, u32x4 (&vf
 #pragma unroll
         for (int db = 0; db < 2; db++) {
             const unsigned char *p =
-                reinterpret_cast<const unsigned char *>((uintptr_t)(t.vlane + (kb * 32 + 16 * h) * 128) ^ (64u * db));
+                HI ? (db ? t.vlane_hi : t.vlane) + (kb * 32 + 16 * h) * 128
+                   : reinterpret_cast<const unsigned char *>((uintptr_t)(t.vlane + (kb * 32 + 16 * h) * 128) ^ (64u * db));
             const u32x2 lo = att_tr_read(p), hi = att_tr_read(p + 8 * 128);
             vf[2 * h + db].x = lo.x;
             vf[2 * h + db].y = lo.y;
@@ -150,13 +156,13 @@ __device__ __forceinline__ float att_max16_if_positive(const f32x16 &s)
 // interleaved with the score MFMAs of block kb+1 (fragments in `kf` -> `sn`, when NEXT); each fragment of K is
 // replaced by that of block kb+2 (when NEXT2) as soon as its MFMA has been issued.  MASK: block kb is the last
 // one and runs past the keys.
-template <bool NEXT, bool NEXT2, bool MASK>
+template <bool NEXT, bool NEXT2, bool MASK, bool HI = false>
 __device__ __forceinline__ void att_step(const AttnTile &t, const int (&cs)[4], int kb, f32x16 &sc, f32x16 &sn,
                                          u32x4 (&kf)[4], const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm,
                                          float (&l)[2])
 {
     u32x4 vf[4];
-    att_read_v(t, kb, vf);
+    att_read_v<HI>(t, kb, vf);
     if constexpr (MASK) {
         const int lim = t.n - kb * 32 - 4 * t.lg;
 #pragma unroll
@@ -331,10 +337,10 @@ __device__ __forceinline__ void att_stage_fixed(const AttnTile &t, const int (&c
         constexpr int kb = decltype(kbc)::value;
         constexpr bool NEXT = kb + 1 < NB, NEXT2 = kb + 2 < NB;
         if constexpr (kb == NB - 1) {
-            if (partial) att_step<NEXT, NEXT2, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
-            else att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            if (partial) att_step<NEXT, NEXT2, true, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            else att_step<NEXT, NEXT2, false, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
         } else {
-            att_step<NEXT, NEXT2, false>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            att_step<NEXT, NEXT2, false, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
         }
     });
 }
@@ -477,7 +483,7 @@ __global__ __launch_bounds__(512, 1) void sparse_attention_bf16_d64_pipelined_ke
             if (wid >= NW / 2) stage_issue(nxt, smem + (par ^ 1) * bufsz, wid - NW / 2, NW / 2);
             load_q(nxt, wid, qn);
         }
-        const AttnTile tile = {buf + lr * 128, att_v_lane(buf + npad * 128, lane), n, lg};
+        const AttnTile tile = {buf + lr * 128, att_v_lane(buf + npad * 128, lane), nullptr, n, lg};
         for (int rt = wid; rt * 32 < cur.Lb; rt += NW) {
             const int qrow = rt * 32 + lr;
             if (rt != wid) {        // a ninth tile and beyond (more than 256 queries): waits behind the prefetch
@@ -601,7 +607,8 @@ __global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_stream_kerne
     const int nfull = n / ASK;                        // stages of four whole blocks; then at most one shorter stage
     auto stage_tile = [&](int st) {
         const unsigned char *buf = smem + (st & 1) * ASBUF;
-        return AttnTile{buf + lr * 128, att_v_lane(buf + ASK * 128, lane), n - st * ASK, lg};
+        const unsigned char *vl = att_v_lane(buf + ASK * 128, lane);
+        return AttnTile{buf + lr * 128, vl, reinterpret_cast<const unsigned char *>((uintptr_t)vl ^ 64u), n - st * ASK, lg};
     };
     for (int st = 0; st < nfull; st++) {
         wait_vmcnt<0>();                 // this wave's loads of stage st (nothing younger is in flight)
