@@ -631,6 +631,34 @@ def test_sparse_attention(dev, dtype, B, h, d, n, lo, hi):
     assert_close(got.float(), want, dtype, "sparse attention")
 
 
+@pytest.mark.parametrize("n", [257, 1025])
+@pytest.mark.parametrize("shape", ["ramp", "late spike", "early spike", "steps"])
+def test_sparse_attention_scores_far_above_the_first_block(dev, n, shape):
+    """The softmax's reference is taken from the first 32 keys and raised on the way: scores that climb steadily
+    (the reference is raised many times), a single key hundreds above all others near the end (more than fp32 can
+    hold as a probability relative to the old reference) or in the first block, and plateaus that jump by 60 between
+    stages of 128 keys.  Both bf16 kernels (keys resident: 257, streamed: 1025) against the oracle's max-subtracted
+    softmax."""
+    from vtpack_amd import _C
+    B, h, d = 3, 2, 64
+    lengths = np.array([130, 33, 70], dtype=np.int64)
+    L = int(lengths.sum())
+    q, k, v = 0.05 * randn(720, h, L, d), 0.05 * randn(721, h, B, n, d), randn(722, h, B, n, d)
+    j = np.arange(n, dtype=np.float32)
+    level = {"ramp": 0.25 * j, "late spike": np.where(j == n - 7, 300.0, 0.0), "early spike": np.where(j == 5, 300.0, 0.0),
+             "steps": 60.0 * np.floor(j / 128)}[shape]
+    q[..., 0] = 8.0                               # times scale = 1/8: a key's score is its level plus noise
+    k[..., 0] = level
+    q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+    scale = d ** -0.5
+    want = orc.attention(q, k, v, lengths, scale)
+    assert np.isfinite(want).all()
+    got = _C.batched_sparse_attention_forward(_t(q, dev, torch.bfloat16), _t(k, dev, torch.bfloat16),
+                                              _t(v, dev, torch.bfloat16), torch.from_numpy(lengths), scale)
+    assert bool(torch.isfinite(got).all())
+    assert_close(got.float(), want, torch.bfloat16, f"sparse attention, {shape} over {n} keys")
+
+
 @pytest.mark.parametrize("n", [20, 32, 64, 96, 128, 160, 192, 196, 256, 257, 288])
 def test_sparse_attention_resident_keys_many_items(dev, n):
     """bf16, head_dim 64, up to 288 keys: the kernel that keeps an item's keys and values in LDS, with more

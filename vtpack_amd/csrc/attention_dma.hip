@@ -10,6 +10,7 @@
 //     direct loads, V through registers and transposed writes, online softmax in the log2 domain.
 #include "common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace vtdge {
 
@@ -156,7 +157,8 @@ __device__ __forceinline__ float att_max16_if_positive(const f32x16 &s)
 // interleaved with the score MFMAs of block kb+1 (fragments in `kf` -> `sn`, when NEXT); each fragment of K is
 // replaced by that of block kb+2 (when NEXT2) as soon as its MFMA has been issued.  MASK: block kb is the last
 // one and runs past the keys.
-template <bool NEXT, bool NEXT2, bool MASK, bool HI = false>
+// FAST: no test of the block's scores against the reference (the caller looks at the row sums once per stage).
+template <bool NEXT, bool NEXT2, bool MASK, bool HI = false, bool FAST = false>
 __device__ __forceinline__ void att_step(const AttnTile &t, const int (&cs)[4], int kb, f32x16 &sc, f32x16 &sn,
                                          u32x4 (&kf)[4], const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm,
                                          float (&l)[2])
@@ -169,8 +171,8 @@ __device__ __forceinline__ void att_step(const AttnTile &t, const int (&cs)[4], 
         for (int e = 0; e < 16; e++)
             if (8 * (e >> 2) + (e & 3) >= lim) sc[e] = -INFINITY;
     }
-    const float mx = att_max16_if_positive(sc);
-    if (__builtin_amdgcn_ballot_w64(mx > ATT_RESCALE) != 0) {      // wave-uniform and rare
+    const float mx = FAST ? 0.f : att_max16_if_positive(sc);
+    if (!FAST && __builtin_amdgcn_ballot_w64(mx > ATT_RESCALE) != 0) {      // wave-uniform and rare
         const float mrow = fmaxf(mx, __shfl_xor(mx, 32, WAVE));     // both lanes of a row decide alike
         const float delta = mrow > ATT_RESCALE ? mrow : 0.f;
         const float alpha = __builtin_amdgcn_exp2f(-delta);
@@ -301,9 +303,19 @@ __device__ __forceinline__ void att_tile_fixed(const AttnTile &t, const int (&cs
 // t.n = keys left from the stage's first one).  `first`: the stage opens the sequence (negm is zero and the row's
 // reference is taken from the stage's first block); otherwise the running reference in negm is carried on.  The
 // last block is masked when t.n < 32 NB.
-template <int NB>
+//
+// FAST: the blocks of the stage run without the per-block test (nine vector instructions a block, a fifth of the
+// softmax's).  Probabilities may then grow past 2^8 - harmless in floating point, values and sums keep their
+// precision - and the stage ends with a look at the row sums instead: past ATT_FAST_LIMIT everything is scaled down
+// by a power of two (exactly) and the reference raised by its exponent; a sum that is no longer below ATT_FAST_OVER
+// (a score more than ~100 above everything before it inside one stage, or an overflow outright) sets `bad`, and the
+// caller runs the whole tile again with the per-block test.
+constexpr float ATT_FAST_LIMIT = 16777216.0f;              // 2^24
+constexpr float ATT_FAST_OVER = 1.2676506e30f;             // 2^100
+template <int NB, bool FAST = false>
 __device__ __forceinline__ void att_stage_fixed(const AttnTile &t, const int (&cs)[4], bool first,
-                                                const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm, float (&l)[2])
+                                                const u32x4 (&qf)[4], f32x16 (&o)[2], f32x16 &negm, float (&l)[2],
+                                                bool *bad = nullptr)
 {
     u32x4 kf[4];
     f32x16 sbuf[2];
@@ -337,12 +349,30 @@ __device__ __forceinline__ void att_stage_fixed(const AttnTile &t, const int (&c
         constexpr int kb = decltype(kbc)::value;
         constexpr bool NEXT = kb + 1 < NB, NEXT2 = kb + 2 < NB;
         if constexpr (kb == NB - 1) {
-            if (partial) att_step<NEXT, NEXT2, true, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
-            else att_step<NEXT, NEXT2, false, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            if (partial) att_step<NEXT, NEXT2, true, true, FAST>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            else att_step<NEXT, NEXT2, false, true, FAST>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
         } else {
-            att_step<NEXT, NEXT2, false, true>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
+            att_step<NEXT, NEXT2, false, true, FAST>(t, cs, kb, sbuf[kb & 1], sbuf[(kb + 1) & 1], kf, qf, o, negm, l);
         }
     });
+    if constexpr (FAST) {
+        const float ls = l[0] + l[1];
+        if (__builtin_amdgcn_ballot_w64(!(ls <= ATT_FAST_LIMIT)) != 0) {         // wave-uniform and rare
+            const float other = __shfl_xor(ls, 32, WAVE);
+            const float mrow = ls > other ? ls : other;                          // both lanes of a row decide alike
+            if (__builtin_amdgcn_ballot_w64(!(ls < ATT_FAST_OVER) || !(other < ATT_FAST_OVER)) != 0) *bad = true;
+            const int k = mrow > ATT_FAST_LIMIT ? __builtin_amdgcn_frexp_expf(mrow) : 0;
+            const float alpha = __builtin_amdgcn_ldexpf(1.0f, -k), delta = (float)k;
+            l[0] *= alpha;
+            l[1] *= alpha;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                o[0][e] *= alpha;
+                o[1][e] *= alpha;
+                negm[e] -= delta;
+            }
+        }
+    }
 }
 
 #undef VT_PIN
@@ -602,31 +632,47 @@ __global__ __launch_bounds__(256, 2) void sparse_attention_bf16_d64_stream_kerne
     for (int s = 0; s < 4; s++) cs[s] = ((2 * s + lg) ^ sw) * 16;
 
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    f32x16 o[2] = {zero, zero}, negm = zero;
-    float l[2] = {0.f, 0.f};
+    f32x16 o[2], negm;
+    float l[2];
     const int nfull = n / ASK;                        // stages of four whole blocks; then at most one shorter stage
     auto stage_tile = [&](int st) {
         const unsigned char *buf = smem + (st & 1) * ASBUF;
         const unsigned char *vl = att_v_lane(buf + ASK * 128, lane);
         return AttnTile{buf + lr * 128, vl, reinterpret_cast<const unsigned char *>((uintptr_t)vl ^ 64u), n - st * ASK, lg};
     };
-    for (int st = 0; st < nfull; st++) {
-        wait_vmcnt<0>();                 // this wave's loads of stage st (nothing younger is in flight)
-        __syncthreads();                 // stage st is complete; the other buffer was last read in iteration st-1
-        if (st + 1 < nstage) issue(st + 1);
-        if (wave_live) att_stage_fixed<4>(stage_tile(st), cs, st == 0, qf, o, negm, l);
-    }
-    if (nfull < nstage) {                // the last, shorter stage: 1 .. 3 blocks (its own code, outside the loop)
-        wait_vmcnt<0>();
-        __syncthreads();
-        if (wave_live) {
-            const AttnTile tile = stage_tile(nfull);
-            switch ((tile.n + 31) / 32) {
-            case 3: att_stage_fixed<3>(tile, cs, nfull == 0, qf, o, negm, l); break;
-            case 2: att_stage_fixed<2>(tile, cs, nfull == 0, qf, o, negm, l); break;
-            default: att_stage_fixed<1>(tile, cs, nfull == 0, qf, o, negm, l); break;
+    // All stages of the sequence (stage 0 is on its way); FAST: see att_stage_fixed.  -> whether a row sum left
+    // the range the fast form is good for.
+    auto all_stages = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        bool bad = false;
+        o[0] = o[1] = negm = zero;
+        l[0] = l[1] = 0.f;
+        for (int st = 0; st < nfull; st++) {
+            wait_vmcnt<0>();                 // this wave's loads of stage st (nothing younger is in flight)
+            __syncthreads();                 // stage st is complete; the other buffer was last read in iteration st-1
+            if (st + 1 < nstage) issue(st + 1);
+            if (wave_live) att_stage_fixed<4, FAST>(stage_tile(st), cs, st == 0, qf, o, negm, l, &bad);
+        }
+        if (nfull < nstage) {                // the last, shorter stage: 1 .. 3 blocks (its own code, outside the loop)
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (wave_live) {
+                const AttnTile tile = stage_tile(nfull);
+                switch ((tile.n + 31) / 32) {
+                case 3: att_stage_fixed<3, FAST>(tile, cs, nfull == 0, qf, o, negm, l, &bad); break;
+                case 2: att_stage_fixed<2, FAST>(tile, cs, nfull == 0, qf, o, negm, l, &bad); break;
+                default: att_stage_fixed<1, FAST>(tile, cs, nfull == 0, qf, o, negm, l, &bad); break;
+                }
             }
         }
+        return bad;
+    };
+    const bool bad = all_stages(std::true_type{});
+    // The keys are staged for the whole workgroup, so a second pass is one for all its waves (their results come out
+    // the same as before); it starts once every wave has left the buffers of the first.
+    if (__syncthreads_or(bad ? 1 : 0)) {
+        issue(0);
+        all_stages(std::false_type{});
     }
     if (!wave_live) return;
     const float l_run = l[0] + l[1];
