@@ -394,9 +394,10 @@ int launch_linear_dma(const void *A, int64_t lda, const void *W, const void *bia
                       hipStream_t st)
 {
     LinArgs a{A, lda, W, bias, res, ldr, out, ldo, rows_dev, rows, N, K, act, st};
-    // wide outputs: 256x128 tiles on 8 MFMA waves; narrow ones (N <= 512): 128x128 on 4, for more tiles.  Other
-    // shapes of the same template (2 loader waves, 128x256 and 128x384 tiles on a two-stage ring) measured no faster.
-    if (N >= 768) return pick_epilogue<T, 256, 128, 4, 2, 4>(a);
+    // wide outputs: 256x128 tiles on 8 MFMA waves; narrow ones (N <= 512), and matrices that have fewer large tiles
+    // than the chip has compute units (a classifier on 256 rows): 128x128 on 4, for more tiles.  Other shapes of the
+    // same template (2 loader waves, 128x256 and 128x384 tiles on a two-stage ring) measured no faster.
+    if (N >= 768 && ceil_div(rows, 256) * ceil_div(N, 128) >= 256) return pick_epilogue<T, 256, 128, 4, 2, 4>(a);
     return pick_epilogue<T, 128, 128, 2, 2, 4>(a);
 }
 
