@@ -256,6 +256,33 @@ def test_deit_small_bf16_model_on_the_weight_stationary_kernels(dev):
     assert_close(got.float(), want, torch.bfloat16, "DeiT-S+DGE bf16 logits, batch 8")
 
 
+def test_scatter_back_that_packs_the_next_block_is_the_same_model(dev):
+    """With and without the scatter-back packing the next block's queries (and with the region kernels off
+    altogether) the model is the same arithmetic on the same rows: logits, gate choices, descriptors and query
+    counts of every block are identical."""
+    from vtpack_amd import engine
+    from vtpack_amd.synthetic import synthetic_images
+    m = _model("deit_dge_s124_small_patch16_256", dev, torch.bfloat16, seed=7)
+    img = synthetic_images(8, 256, seed=8, dtype=torch.bfloat16).to(dev)
+
+    def run():
+        with torch.no_grad():
+            out = m(img)
+        return out, [(b.dge.states["gate"].clone(), b.dge.states["patches"].clone(), b.dge.states["batches"].clone(),
+                      b.dge.states["comp"].clone()) for b in m.blocks]
+
+    chained, st_chained = run()
+    engine.PACK_NEXT = False
+    try:
+        apart, st_apart = run()
+    finally:
+        engine.PACK_NEXT = True
+    assert torch.equal(chained, apart)
+    for a, b in zip(st_chained, st_apart):
+        for u, v in zip(a, b):
+            assert torch.equal(u, v)
+
+
 @pytest.mark.parametrize("factory,heads", [("deit_dge_s124_base_patch16_256", 12), ("deit_dge_s124_tiny_patch16_256", 3)])
 def test_deit_other_widths_bf16_model(dev, factory, heads):
     """The other widths the reference ships (DeiT-Base: 768 channels, 12 heads; DeiT-Ti: 192 channels, 3 heads;
