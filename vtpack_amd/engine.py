@@ -1,17 +1,19 @@
 """Fused inference path of one DGE transformer block: every step on libvtdge kernels.
 
 What `Block.forward` of the reference does with ~30 library launches and one device->host copy
-(vtpack/models/dge/deit_dge.py:123-130) becomes 9 kernel launches (on two streams, joined before attention) with the
-packed query count kept in device memory: buffers are sized for the worst case (one query per
-token) and every packed kernel reads the live row count itself.  Nothing here synchronises, so the
-whole forward can be captured into a HIP graph.
+(vtpack/models/dge/deit_dge.py:123-130) becomes six kernel launches on the caller's stream where the weight-stationary
+and region kernels apply (bf16, 384 channels: key/value + query projection, attention, output projection, fc1, fc2,
+and a scatter-back that also routes and packs the next block), nine on two streams joined before attention
+elsewhere, with the packed query count kept in device memory: buffers are sized for the worst case (one query per
+token) and every packed kernel reads the live row count itself.  Nothing here synchronises, so the whole forward can
+be captured into a HIP graph.
 """
 import torch
 
 from . import ops
 from .layers.dge import Deferred
 
-# The block has two independent chains before attention: the routing chain (router -> index->patch -> compress ->
+# Where the block runs on two streams, it has two independent chains before attention: the routing chain (router -> index->patch -> compress ->
 # q projection: small, latency-bound launches) and the key/value chain (LayerNorm of all tokens -> kv projection:
 # the largest GEMM).  They are issued on two HIP streams of equal (default) priority and joined before attention,
 # in eager mode and inside a captured graph alike.
