@@ -240,6 +240,13 @@ int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t 
                            int64_t *offsets, int64_t *lengths, int32_t *region_rows, int B, int H, int W, int C,
                            int extra, int R, int S, int dtype, void *stream);
 
+/* vtdge_layernorm followed by the addition of a periodic set of rows: out[r] = LayerNorm(x[r]) + add[r mod add_rows],
+ * the LayerNorm's result rounded to the storage type before the addition as the two modules would.  Stands in for a
+ * patch embedding's norm followed by `x + pos_embed` (vtpack/models/dge/pvt_dge.py:176 with :312-314; add =
+ * pos_embed [H*W, C], rows = B * H*W). */
+int vtdge_layernorm_add(const void *x, const void *weight, const void *bias, const void *add, int64_t add_rows,
+                        void *out, int64_t rows, int C, float eps, int dtype, void *stream);
+
 /* Row-wise LayerNorm over the last dimension (biased variance, fp32 statistics).
  * Stands in for nn.LayerNorm(eps=1e-6) at vtpack/models/dge/deit_dge.py:127-128. */
 int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out, const int64_t *rows_dev,

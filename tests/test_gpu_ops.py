@@ -346,6 +346,23 @@ def test_layernorm(dev, dtype, rows, C):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,period,C", [(4096, 1024, 64), (1537, 29, 384), (640, 64, 512), (300, 300, 768)])
+def test_layernorm_with_rows_added(dev, dtype, rows, period, C):
+    """LayerNorm followed by `+ pos_embed` in one pass: bit for bit the LayerNorm kernel's result plus the addend
+    (rounded in between as the two modules would round), for row counts that are and are not multiples of the period."""
+    from vtpack_amd import ops
+    g = torch.Generator().manual_seed(rows + C)
+    x = (torch.randn(rows, C, generator=g) * 2 + 1).to(dtype).to(dev)
+    w = (1 + 0.2 * torch.randn(C, generator=g)).to(dtype).to(dev)
+    b = (0.1 * torch.randn(C, generator=g)).to(dtype).to(dev)
+    pos = torch.randn(1, period, C, generator=g).to(dtype).to(dev)
+    want = ops.layernorm(x, w, b, 1e-6)
+    want = want + pos[0][torch.arange(rows, device=dev) % period]
+    got = ops.layernorm(x, w, b, 1e-6, add=pos)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("B,N,C,count", [(256, 257, 384, 1), (5, 66, 192, 2), (3, 17, 768, 17), (9, 10, 64, 3)])
 def test_layernorm_of_the_front_rows(dev, dtype, B, N, C, count):
     """The final norm on the class-token rows only, read in place: the same bits as LayerNorm of a copy of the slice."""

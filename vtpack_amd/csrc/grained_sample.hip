@@ -1266,8 +1266,11 @@ template <typename T, int NIT, int GS>   // NIT = 16-byte vectors per lane = cei
 __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                          const T *__restrict__ bsrc, T *__restrict__ out,
                                                          const int64_t *__restrict__ rows_dev, int64_t rows, int C,
-                                                         float eps, int64_t x_group_stride, int x_group_rows)
+                                                         float eps, int64_t x_group_stride, int x_group_rows,
+                                                         const T *__restrict__ add = nullptr, int64_t add_rows = 1)
 {
+    // add (nullable) [add_rows, C]: row (r mod add_rows) of it is added to output row r after that row's rounding to
+    // the storage type, and the sum rounded again - a LayerNorm module followed by `+ pos_embed`.
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & (GS - 1);
     const int64_t live = live_rows(rows_dev, rows);
@@ -1328,6 +1331,13 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
                 float y[VEC];
 #pragma unroll
                 for (int c = 0; c < VEC; c++) y[c] = (vals[it][c] - mean) * rstd * ww[it][c] + bb[it][c];
+                if (add != nullptr) {
+                    float a[VEC];
+                    Elem<T>::unpack(*reinterpret_cast<const u32x4 *>(add + ((row0 + r) % add_rows) * C + v * VEC), a);
+                    Elem<T>::unpack(Elem<T>::pack(y), y);
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) y[c] += a[c];
+                }
                 *reinterpret_cast<u32x4 *>(out + (row0 + r) * (int64_t)C + v * VEC) = Elem<T>::pack(y);
             }
         }
@@ -1881,7 +1891,15 @@ extern "C" int vtdge_router_stats(void *x, const void *front_rows, const void *w
 
 static int layernorm_launch(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight,
                             const void *bias, void *out, const int64_t *rows_dev, int64_t rows, int C, float eps,
-                            int dtype, void *stream);
+                            int dtype, void *stream, const void *add = nullptr, int64_t add_rows = 1);
+
+extern "C" int vtdge_layernorm_add(const void *x, const void *weight, const void *bias, const void *add,
+                                   int64_t add_rows, void *out, int64_t rows, int C, float eps, int dtype,
+                                   void *stream)
+{
+    VT_REQUIRE(add != nullptr, VTDGE_ERR_ARG, "layernorm_add: NULL operand");
+    return layernorm_launch(x, 0, 0, weight, bias, out, nullptr, rows, C, eps, dtype, stream, add, add_rows);
+}
 
 extern "C" int vtdge_layernorm(const void *x, const void *weight, const void *bias, void *out,
                                const int64_t *rows_dev, int64_t rows, int C, float eps, int dtype, void *stream)
@@ -1902,9 +1920,11 @@ extern "C" int vtdge_layernorm_rows(const void *x, int64_t x_group_stride, int x
 
 static int layernorm_launch(const void *x, int64_t x_group_stride, int x_group_rows, const void *weight,
                             const void *bias, void *out, const int64_t *rows_dev, int64_t rows, int C, float eps,
-                            int dtype, void *stream)
+                            int dtype, void *stream, const void *add, int64_t add_rows)
 {
     VT_REQUIRE(x && weight && bias && out, VTDGE_ERR_ARG, "layernorm: NULL operand");
+    VT_REQUIRE(add == nullptr || (add_rows > 0 && aligned16(add)), VTDGE_ERR_ARG,
+               "layernorm: the rows to add need a positive count and 16-byte alignment");
     VT_REQUIRE(rows >= 0, VTDGE_ERR_ARG, "layernorm: negative rows");
     if (int rc = check_channels(C, dtype, "layernorm")) return rc;
     const int vec = dtype == VTDGE_BF16 ? 8 : 4;
@@ -1920,7 +1940,8 @@ static int layernorm_launch(const void *x, int64_t x_group_stride, int x_group_r
 #define VT_LAUNCH(T, NIT, GS)                                                                                        \
     note_kernel(reinterpret_cast<const void *>(layernorm_kernel<T, NIT, GS>)),                                       \
     layernorm_kernel<T, NIT, GS><<<grid, block, 0, st>>>((const T *)x, (const T *)weight, (const T *)bias, (T *)out, \
-                                                         rows_dev, rows, C, eps, x_group_stride, x_group_rows)
+                                                         rows_dev, rows, C, eps, x_group_stride, x_group_rows,       \
+                                                         (const T *)add, add_rows)
 #define VT_GROUP(T)                                                                                       \
     do {                                                                                                  \
         if (gs == 64) { if (nit == 1) VT_LAUNCH(T, 1, 64); else if (nit == 2) VT_LAUNCH(T, 2, 64); else VT_LAUNCH(T, 3, 64); } \

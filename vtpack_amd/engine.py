@@ -490,8 +490,13 @@ def pvt_forward(model, images):
             tok = _strided_conv(x, H, W, k, pe.proj)
             H, W = H // k, W // k
         C = tok.shape[-1]
-        tok = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps).view(B, H * W, C)
         last = i == model.num_stages - 1
+        if not last:
+            # the patch embedding's norm and `+ pos_embed` in one pass
+            x = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps,
+                              add=model._get_pos_embed(pos, pe, H, W)).view(B, H * W, C)
+        else:
+            tok = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps).view(B, H * W, C)
         if last:
             x = torch.empty((B, 1 + H * W, C), dtype=tok.dtype, device=tok.device)
             x[:, 1:, :] = tok
@@ -499,8 +504,6 @@ def pvt_forward(model, images):
             if H * W != pe.num_patches:
                 pos = torch.cat((pos[:, :1], model._get_pos_embed(pos[:, 1:], pe, H, W)), dim=1)
             x += pos
-        else:
-            x = tok + model._get_pos_embed(pos, pe, H, W)
         x = _run_blocks(list(getattr(model, f"block{i + 1}")), x, H, W)
         if not last:
             outputs[f"res{i + 2}"] = x.view(B, H, W, C)

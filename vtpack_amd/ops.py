@@ -409,8 +409,10 @@ def fits_decompress_layernorm(x):
     return x.shape[-1] * x.element_size() <= 64 * 16
 
 
-def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
-    _need_gpu(x, weight, bias)
+def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None, add=None):
+    """LayerNorm over the last dimension.  `add` [P, C] (e.g. a position embedding): row r of the result also gets row
+    r mod P of it, added after the LayerNorm's rounding to the storage type as `norm(x) + pos` would."""
+    _need_gpu(x, weight, bias, add)
     x = _contig(x)
     C = x.shape[-1]
     _check_like(x, weight=weight, bias=bias, out=out)
@@ -422,6 +424,14 @@ def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None):
         out = torch.empty_like(x)
     elif out.shape != x.shape or not out.is_contiguous():
         raise ValueError("out must be a contiguous tensor of the input's shape")
+    if add is not None:
+        if rows_dev is not None:
+            raise ValueError("layernorm: `add` goes with all rows (no live row count)")
+        _check_like(x, add=add)
+        add = _contig(add.reshape(-1, C))
+        call("vtdge_layernorm_add", ptr(x), ptr(weight), ptr(bias), ptr(add), add.shape[0], ptr(out), rows, C,
+             float(eps), dtype_code(x), stream_ptr(), tag=("layernorm", False, rows, C))
+        return out
     call("vtdge_layernorm", ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(rows_dev), rows, C, float(eps),
          dtype_code(x), stream_ptr(), tag=("layernorm", rows_dev is not None, rows, C))
     return out
