@@ -240,6 +240,17 @@ int vtdge_compress_regions(const void *x, const int64_t *indices, const int64_t 
                            int64_t *offsets, int64_t *lengths, int32_t *region_rows, int B, int H, int W, int C,
                            int extra, int R, int S, int dtype, void *stream);
 
+/* The patch embedding of a pyramid model's first stage in one pass over the images: Conv2d(Cin, N, kernel P, stride P)
+ * + bias, the embedding's LayerNorm and `+ pos_embed` (vtpack/models/dge/pvt_dge.py:143-176 with :312-314), each
+ * rounded to the storage type as the separate modules would round.
+ *   images [B, Cin, S, S]   weight [N, Cin*P*P] (the convolution's weight, flattened)   bias, ln_weight, ln_bias [N]
+ *   pos (nullable) [(S/P)^2, N]   out [B * (S/P)^2, N]
+ * bf16, Cin = 3, P = 4, N = 64, S a multiple of 64; VTDGE_ERR_UNSUPPORTED otherwise (the caller then gathers the patches
+ * and uses vtdge_linear, vtdge_layernorm_add). */
+int vtdge_patch_embed_norm(const void *images, const void *weight, const void *bias, const void *ln_weight,
+                           const void *ln_bias, float ln_eps, const void *pos, void *out, int B, int Cin, int S, int P,
+                           int N, int dtype, void *stream);
+
 /* vtdge_layernorm followed by the addition of a periodic set of rows: out[r] = LayerNorm(x[r]) + add[r mod add_rows],
  * the LayerNorm's result rounded to the storage type before the addition as the two modules would.  Stands in for a
  * patch embedding's norm followed by `x + pos_embed` (vtpack/models/dge/pvt_dge.py:176 with :312-314; add =

@@ -141,3 +141,46 @@ def test_pvt_feature_maps(dev):
     for name, c, s in (("res2", 64, 32), ("res3", 128, 16), ("res4", 320, 8), ("res5", 512, 4)):
         assert tuple(fused[name].shape) == (2, c, s, s)
         assert rel_err(fused[name], layer[name].cpu()) <= FP32_REL
+
+
+@pytest.mark.parametrize("B,S,with_pos", [(2, 64, True), (3, 256, True), (1, 128, False)])
+def test_first_stage_patch_embedding_in_one_pass(dev, B, S, with_pos):
+    """Conv2d(3, 64, 4, 4) + bias, LayerNorm and `+ pos_embed` as one kernel (bf16): against torch in fp64 on the same
+    bf16 operands, and against the three-launch composition it replaces (gathered patches -> Linear -> LayerNorm with
+    the addend), from which it may differ by a rounding step where an fp32 sum falls next to a tie."""
+    from vtpack_amd import ops
+    g = torch.Generator().manual_seed(S + B)
+    img = torch.randn(B, 3, S, S, generator=g).bfloat16().to(dev)
+    conv_w = (torch.randn(64, 3, 4, 4, generator=g) * 0.2).bfloat16().to(dev)
+    conv_b = (torch.randn(64, generator=g) * 0.1).bfloat16().to(dev)
+    ln_w = (1 + 0.2 * torch.randn(64, generator=g)).bfloat16().to(dev)
+    ln_b = (0.1 * torch.randn(64, generator=g)).bfloat16().to(dev)
+    G = S // 4
+    pos = (torch.randn(1, G * G, 64, generator=g) * 0.5).bfloat16().to(dev) if with_pos else None
+    assert ops.fits_patch_embed_norm(img, conv_w, 4)
+    got = ops.patch_embed_norm(img, conv_w, conv_b, ln_w, ln_b, 1e-6, pos, 4)
+    assert got.shape == (B, G * G, 64)
+    # fp64 statement of the modules, rounded to bf16 where they would round
+    y = torch.nn.functional.conv2d(img.double(), conv_w.double(), conv_b.double(), stride=4)
+    y = y.flatten(2).transpose(1, 2).bfloat16().double()
+    y = torch.nn.functional.layer_norm(y, (64,), ln_w.double(), ln_b.double(), 1e-6).bfloat16().double()
+    want = (y + pos.double()).bfloat16() if with_pos else y.bfloat16()
+    err = (got.double() - want.double()).abs()
+    assert float((err / want.double().abs().clamp_min(1.0)).max()) <= 2.0 ** -6          # at most two bf16 steps
+    assert float((err > 0).double().mean()) < 0.03
+    # the composition it replaces
+    pat = img.reshape(B, 3, G, 4, G, 4).permute(0, 2, 4, 1, 3, 5).reshape(B * G * G, 48)
+    tok = ops.linear(pat, conv_w.reshape(64, 48), conv_b)
+    ref = ops.layernorm(tok, ln_w, ln_b, 1e-6, add=pos) if with_pos else ops.layernorm(tok, ln_w, ln_b, 1e-6)
+    d = (got.float() - ref.view(B, G * G, 64).float()).abs()
+    assert float((d / ref.view(B, G * G, 64).float().abs().clamp_min(1.0)).max()) <= 2.0 ** -6
+    assert float((d > 0).float().mean()) < 0.03
+
+
+def test_first_stage_patch_embedding_refuses_other_shapes(dev):
+    from vtpack_amd import ops
+    img = torch.zeros(1, 3, 96, 96, dtype=torch.bfloat16, device=dev)            # side not a multiple of 64
+    w = torch.zeros(64, 3, 4, 4, dtype=torch.bfloat16, device=dev)
+    assert not ops.fits_patch_embed_norm(img, w, 4)
+    assert not ops.fits_patch_embed_norm(img.float(), w.float(), 4)
+    assert not ops.fits_patch_embed_norm(torch.zeros(1, 3, 64, 64, dtype=torch.bfloat16, device=dev), w[:32], 4)

@@ -43,6 +43,7 @@ SIGNATURES = {
     "vtdge_router_stats": [_p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_compress_regions": [_p, _p, _p, _p, _p, _p, _f, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_layernorm": [_p, _p, _p, _p, _p, _l, _i, _f, _i, _p],
+    "vtdge_patch_embed_norm": [_p, _p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _p],
     "vtdge_layernorm_add": [_p, _p, _p, _p, _l, _p, _l, _i, _f, _i, _p],
     "vtdge_layernorm_rows": [_p, _l, _i, _p, _p, _p, _l, _i, _f, _i, _p],
     "vtdge_linear": [_p, _l, _p, _p, _p, _l, _p, _l, _p, _l, _i, _i, _i, _i, _p],

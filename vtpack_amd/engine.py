@@ -479,23 +479,34 @@ def pvt_forward(model, images):
         pe = getattr(model, f"patch_embed{i + 1}")
         pos = getattr(model, f"pos_embed{i + 1}")
         k = pe.patch_size[0]
+        last = i == model.num_stages - 1
+        tok = None
         if i == 0:
             H, W = Hi // k, Wi // k
-            pat = images[:, :, :H * k, :W * k].reshape(B, Cin, H, k, W, k).permute(0, 2, 4, 1, 3, 5)
-            tok = ops.linear(pat.reshape(B * H * W, Cin * k * k), pe.proj.weight.reshape(pe.proj.weight.shape[0], -1),
-                             pe.proj.bias)
+            if (FUSE_PATCH_EMBED and not last and Hi == Wi and H * W == pe.num_patches
+                    and ops.fits_patch_embed_norm(images, pe.proj.weight, k)):
+                # convolution, the embedding's LayerNorm and the position embedding in one pass over the images
+                x = ops.patch_embed_norm(images, pe.proj.weight, pe.proj.bias, pe.norm.weight, pe.norm.bias,
+                                         pe.norm.eps, pos, k)
+                C = x.shape[-1]
+            else:
+                pat = images[:, :, :H * k, :W * k].reshape(B, Cin, H, k, W, k).permute(0, 2, 4, 1, 3, 5)
+                tok = ops.linear(pat.reshape(B * H * W, Cin * k * k),
+                                 pe.proj.weight.reshape(pe.proj.weight.shape[0], -1), pe.proj.bias)
         else:
             if H % k or W % k:
                 raise ValueError(f"token grid {H}x{W} is not a multiple of the stage's patch size {k}")
             tok = _strided_conv(x, H, W, k, pe.proj)
             H, W = H // k, W // k
-        C = tok.shape[-1]
-        last = i == model.num_stages - 1
-        if not last:
+        if tok is None:
+            pass
+        elif not last:
             # the patch embedding's norm and `+ pos_embed` in one pass
+            C = tok.shape[-1]
             x = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps,
                               add=model._get_pos_embed(pos, pe, H, W)).view(B, H * W, C)
         else:
+            C = tok.shape[-1]
             tok = ops.layernorm(tok, pe.norm.weight, pe.norm.bias, pe.norm.eps).view(B, H * W, C)
         if last:
             x = torch.empty((B, 1 + H * W, C), dtype=tok.dtype, device=tok.device)

@@ -409,6 +409,34 @@ def fits_decompress_layernorm(x):
     return x.shape[-1] * x.element_size() <= 64 * 16
 
 
+def fits_patch_embed_norm(images, weight, P):
+    """Whether `patch_embed_norm` has a kernel: bf16 images of 3 channels, 4 x 4 patches, 64 outputs, a side that is a
+    multiple of 64."""
+    return (images.is_cuda and images.dtype == torch.bfloat16 and images.dim() == 4 and images.shape[1] == 3 and P == 4
+            and weight.shape[0] == 64 and images.shape[2] == images.shape[3] and images.shape[2] % 64 == 0
+            and images.is_contiguous())
+
+
+def patch_embed_norm(images, weight, bias, ln_weight, ln_bias, ln_eps, pos, P):
+    """images [B, 3, S, S] -> tokens [B, (S/P)^2, N]: the stride-P convolution (weight [N, 3, P, P]) + bias, LayerNorm
+    and `+ pos` [(S/P)^2, N] (optional) in one pass.  See `fits_patch_embed_norm`."""
+    _need_gpu(images, weight, bias, ln_weight, ln_bias, pos)
+    B, Cin, S, _ = images.shape
+    N = weight.shape[0]
+    G = S // P
+    _check_like(images, weight=weight, bias=bias, ln_weight=ln_weight, ln_bias=ln_bias, pos=pos)
+    w2 = _contig(weight.reshape(N, Cin * P * P))
+    if pos is not None:
+        pos = _contig(pos.reshape(-1, N))
+        if pos.shape[0] != G * G:
+            raise ValueError(f"pos holds {pos.shape[0]} rows, the grid has {G * G} patches")
+    out = torch.empty((B, G * G, N), dtype=images.dtype, device=images.device)
+    call("vtdge_patch_embed_norm", ptr(images), ptr(w2), ptr(_contig(bias)), ptr(_contig(ln_weight)),
+         ptr(_contig(ln_bias)), float(ln_eps), ptr(pos), ptr(out), B, Cin, S, P, N, dtype_code(images), stream_ptr(),
+         tag=("patch_embed_norm", B, S))
+    return out
+
+
 def layernorm(x, weight, bias, eps=1e-6, rows_dev=None, out=None, add=None):
     """LayerNorm over the last dimension.  `add` [P, C] (e.g. a position embedding): row r of the result also gets row
     r mod P of it, added after the LayerNorm's rounding to the storage type as `norm(x) + pos` would."""
